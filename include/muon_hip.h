@@ -1,0 +1,143 @@
+/* C ABI of libmuon_hip.so: the Muon optimizer step of lmms-engine on one MI355X (gfx950).
+ *
+ * The reference path is pure Python (src/lmms_engine/utils/muon_utils.py); its "FFI" is the
+ * set of torch / Triton calls that file makes.  Each entry point below replaces one group of
+ * those calls, cited as muon_utils.py:LINE.  A Python caller binds them with ctypes
+ * (lmms_engine_amd/_abi.py); any other host can bind the same symbols.
+ *
+ * Conventions
+ *  - Plain C types only.  Device pointers are borrowed for the duration of the call; the
+ *    library never allocates, frees or retains device memory.
+ *  - `stream` is a hipStream_t (0 = the null stream).  Every call only enqueues work on it
+ *    and returns without synchronising the host.
+ *  - Return value: 0 on success, a positive hipError_t when the runtime failed, a negative
+ *    MUON_HIP_E* code when an argument was rejected.  muon_hip_last_error() describes the
+ *    last failure on the calling thread.
+ *  - dtype codes: MUON_HIP_F32 = 0, MUON_HIP_BF16 = 1.
+ *  - A parameter is `rows x cols`, row-major, contiguous.  M = min(rows, cols),
+ *    K = max(rows, cols); "transposed" means rows > cols (muon_utils.py:139-140).
+ *  - Batched entry points work on `batch` matrices of one shape.  Optimizer tensors are
+ *    reached through device-resident pointer tables (`const void* const*`, `batch` entries).
+ *  - The Newton-Schulz operands live in a caller-allocated workspace of
+ *    muon_hip_workspace_bytes() bytes, 256-byte aligned, which the entry points partition
+ *    identically; its contents between calls are private to the library.
+ */
+#ifndef MUON_HIP_H
+#define MUON_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MUON_HIP_F32 0
+#define MUON_HIP_BF16 1
+
+#define MUON_HIP_EINVAL (-1)  /* bad argument (null pointer, non-positive size, unknown dtype/config) */
+#define MUON_HIP_ESHAPE (-2)  /* shape is not a whole number of tiles / exceeds a launch limit */
+
+/* kernel ids for muon_hip_timing_read */
+#define MUON_HIP_K_MOMENTUM 0
+#define MUON_HIP_K_NORMALIZE 1
+#define MUON_HIP_K_SYRK 2
+#define MUON_HIP_K_SYMPOLY 3
+#define MUON_HIP_K_BX 4
+#define MUON_HIP_K_UPDATE 5
+#define MUON_HIP_K_ADAMW 6
+#define MUON_HIP_K_COUNT 7
+
+/* GEMM tile configurations; MUON_HIP_CFG_AUTO picks by shape. */
+#define MUON_HIP_CFG_AUTO (-1)
+#define MUON_HIP_CFG_128x128_W4 0
+#define MUON_HIP_CFG_256x256_W4 1
+#define MUON_HIP_CFG_256x256_W8 2
+
+int muon_hip_version(void);
+const char* muon_hip_last_error(void);
+
+/* Padded operand geometry for a rows x cols parameter: M, K as above, Mp/Kp the zero-padded
+ * sizes the GEMM kernels work on, tile the square tile edge.  Any out pointer may be null. */
+int muon_hip_geometry(int rows, int cols, int* M, int* K, int* Mp, int* Kp, int* tile);
+
+/* Bytes of workspace one bucket of `batch` rows x cols matrices needs. */
+size_t muon_hip_workspace_bytes(int rows, int cols, int batch);
+
+/* Force one tile configuration for every later call (MUON_HIP_CFG_AUTO restores the default).
+ * Affects geometry and workspace size; meant for benchmarking sweeps. */
+int muon_hip_set_gemm_config(int cfg);
+
+/* ---- stage entry points (workspace based) ------------------------------------------- */
+
+/* muon_update's momentum stage, muon_utils.py:188-189, fused with X = G.bfloat16() (:138)
+ * and the sum of squares behind X.norm (:146):
+ *   m <- lerp(m, g, 1-beta);  u <- nesterov ? lerp(g, m, beta) : m;  workspace.U <- bf16(u)
+ * g is read through g_ptrs (dtype g_dtype), m updated in place through m_ptrs (m_dtype).
+ * Supported (g, m) dtypes: (f32, f32), (bf16, bf16) as the reference, and (bf16, f32).
+ * write_back_grad != 0 also stores u into g, as the reference's in-place lerp_ does. */
+int muon_hip_momentum_norm(const void* const* g_ptrs, const void* const* m_ptrs, int g_dtype, int m_dtype,
+                           void* workspace, int rows, int cols, int batch, double beta, int nesterov,
+                           int write_back_grad, void* stream);
+
+/* The same first stage for fast_newtonschulz called on its own (muon_utils.py:138,146):
+ * G is a dense [batch][rows][cols] tensor; workspace.U <- bf16(G) plus the partial sums. */
+int muon_hip_cast_norm(const void* G, int g_dtype, void* workspace, int rows, int cols, int batch, void* stream);
+
+/* fast_newtonschulz, muon_utils.py:139-156, on what the first stage left in the workspace:
+ * normalise by bf16(bf16(||X||_F) + 1e-7), then `steps` iterations of
+ *   A = X Xt; B = b A + c A A; X = a X + B X
+ * with the reference's bf16 rounding points.  The result stays in the workspace. */
+int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int steps, double a, double b, double c,
+                        void* stream);
+
+/* apply_scaling (muon_utils.py:167-175) and the parameter update (:324-325):
+ *   o = bf16(O * scale);  p <- p * (1 - lr*wd);  p <- p + (-lr) * o
+ * O is the result muon_hip_ns_grouped(steps) left in the workspace.  `scale` is the python
+ * double the reference multiplies by (0.2*sqrt(max(rows, cols)) or sqrt(max(1, rows/cols))). */
+int muon_hip_apply_update(const void* const* p_ptrs, int p_dtype, void* workspace, int rows, int cols, int batch,
+                          int steps, double scale, double lr, double weight_decay, void* stream);
+
+/* Copies the NS result out of the workspace into a dense bf16 [batch][rows][cols] tensor:
+ * the return value of fast_newtonschulz (muon_utils.py:154-156). */
+int muon_hip_ns_output(void* workspace, int rows, int cols, int batch, int steps, void* out, void* stream);
+
+/* The whole Muon step for one bucket: SingelDeviceWork.start (muon_utils.py:315-325) for
+ * `batch` same-shape parameters in one grouped dispatch per stage. */
+int muon_hip_step_grouped(const void* const* p_ptrs, const void* const* g_ptrs, const void* const* m_ptrs,
+                          int p_dtype, int g_dtype, int m_dtype, void* workspace, int rows, int cols, int batch,
+                          double lr, double weight_decay, double beta, int nesterov, int ns_steps, double scale,
+                          double a, double b, double c, int write_back_grad, void* stream);
+
+/* ---- single GEMM entry points (explicit buffers, already padded to whole tiles) ------- */
+
+/* A[batch][Mp][Mp] = bf16(X Xt) for X[batch][Mp][Kp]: matmul_transpose_assign + mmt_kernel,
+ * muon_utils.py:95-119 and :28-92.  Upper tiles computed, mirrored below the diagonal. */
+int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* stream);
+
+/* B = bf16(bf16(b*A) + bf16(c*bf16(A A))) for symmetric A: muon_utils.py:150-151. */
+int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* stream);
+
+/* X' = bf16(bf16(a*X) + bf16(B X)): muon_utils.py:152.  B[batch][Mp][Mp] symmetric,
+ * XT[batch][Kp][Mp] the transposed copy of X; writes Xout[batch][Mp][Kp] and/or
+ * XTout[batch][Kp][Mp] (either may be null, not both). */
+int muon_hip_bx_axpy_bf16(const void* B, const void* XT, void* Xout, void* XTout, int Mp, int Kp, int batch,
+                          double a, int cfg, void* stream);
+
+/* ---- AdamW fallback ------------------------------------------------------------------ */
+
+/* adam_update + the Adam branch of step_fsdp, muon_utils.py:178-183 and :468-477, for one
+ * tensor of n elements; p, g, exp_avg, exp_avg_sq share `dtype`; `step` is already incremented. */
+int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int dtype, long n, int step, double lr,
+                   double beta1, double beta2, double eps, double weight_decay, void* stream);
+
+/* ---- per-kernel timing ----------------------------------------------------------------
+ * No counterpart in the reference.  When enabled, every kernel launch is bracketed by a pair
+ * of HIP events on its own stream; muon_hip_timing_read waits for them and returns the summed
+ * duration and launch count of one kernel id since timing was enabled. */
+int muon_hip_timing_enable(int on);
+int muon_hip_timing_read(int kernel_id, double* total_ms, long* launches);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MUON_HIP_H */

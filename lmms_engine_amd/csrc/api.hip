@@ -1,0 +1,413 @@
+// C ABI of libmuon_hip.so (declared in include/muon_hip.h): argument checks, workspace
+// partitioning, the grouped launch sequence of one Muon step, and per-kernel event timing.
+#include <stdarg.h>
+#include <stdio.h>
+#include <mutex>
+#include <vector>
+
+#include "../../include/muon_hip.h"
+#include "common.h"
+#include "elementwise.h"
+#include "gemm_nt.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+int g_forced_cfg = MUON_HIP_CFG_AUTO;
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+    return (int)e;
+}
+
+// ---- timing ------------------------------------------------------------------------
+struct EventPair {
+    hipEvent_t start, stop;
+};
+std::mutex g_tmu;
+bool g_timing = false;
+std::vector<EventPair> g_events[MUON_HIP_K_COUNT];
+constexpr size_t kMaxEventsPerKernel = 1 << 16;
+
+void clear_events() {
+    for (auto& v : g_events) {
+        for (auto& p : v) {
+            (void)hipEventDestroy(p.start);
+            (void)hipEventDestroy(p.stop);
+        }
+        v.clear();
+    }
+}
+
+struct Timed {
+    int kid;
+    hipStream_t s;
+    EventPair ev;
+    bool on;
+    Timed(int k, hipStream_t st) : kid(k), s(st), on(false) {
+        if (!g_timing) return;
+        std::lock_guard<std::mutex> lk(g_tmu);
+        if (g_events[kid].size() >= kMaxEventsPerKernel) return;
+        if (hipEventCreate(&ev.start) != hipSuccess) return;
+        if (hipEventCreate(&ev.stop) != hipSuccess) {
+            (void)hipEventDestroy(ev.start);
+            return;
+        }
+        on = hipEventRecord(ev.start, s) == hipSuccess;
+    }
+    ~Timed() {
+        if (!on) return;
+        (void)hipEventRecord(ev.stop, s);
+        std::lock_guard<std::mutex> lk(g_tmu);
+        g_events[kid].push_back(ev);
+    }
+};
+
+// ---- geometry / workspace ------------------------------------------------------------
+struct Plan {
+    int rows, cols, batch, M, K, Mp, Kp, tile, cfg, nparts;
+    bool transposed;
+    long n, strideU, strideX, strideA;
+    size_t offX[2], offXT[2], offA, offB, offParts, total;
+};
+
+inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
+
+int pick_cfg(int M) {
+    if (g_forced_cfg != MUON_HIP_CFG_AUTO) return g_forced_cfg;
+    return (M % 256 == 0 && M >= 512) ? GEMM_CFG_256x256_W8 : GEMM_CFG_128x128_W4;
+}
+
+int make_plan(int rows, int cols, int batch, Plan& p) {
+    if (rows <= 0 || cols <= 0 || batch <= 0) return fail(MUON_HIP_EINVAL, "rows, cols and batch must be positive");
+    if (batch > 65535) return fail(MUON_HIP_ESHAPE, "batch %d exceeds 65535 matrices per call", batch);
+    p.rows = rows;
+    p.cols = cols;
+    p.batch = batch;
+    p.transposed = rows > cols;
+    p.M = rows < cols ? rows : cols;
+    p.K = rows < cols ? cols : rows;
+    p.cfg = pick_cfg(p.M);
+    p.tile = gemm_cfg_tile(p.cfg);
+    if (p.tile == 0) return fail(MUON_HIP_EINVAL, "unknown GEMM configuration %d", p.cfg);
+    p.Mp = (int)round_up(p.M, p.tile);
+    p.Kp = (int)round_up(p.K, p.tile);
+    p.n = (long)rows * cols;
+    p.strideU = round_up(p.n, 8);
+    p.strideX = (long)p.Mp * p.Kp;
+    p.strideA = (long)p.Mp * p.Mp;
+    p.nparts = momentum_parts(p.n);
+    const long T = p.Mp / p.tile, TN = p.Kp / p.tile;
+    if (T * TN * batch > 0x7fffffffL) return fail(MUON_HIP_ESHAPE, "too many tiles for one launch");
+    size_t off = 0;
+    auto seg = [&](size_t bytes) {
+        size_t o = off;
+        off += (size_t)round_up((long)bytes, 256);
+        return o;
+    };
+    const size_t xb = (size_t)batch * p.strideX * 2, ab = (size_t)batch * p.strideA * 2;
+    p.offX[0] = seg(xb);
+    p.offX[1] = seg(xb);  // doubles as U (the blend in the parameter's layout) before the first iteration
+    p.offXT[0] = seg(xb);
+    p.offXT[1] = seg(xb);
+    p.offA = seg(ab);
+    p.offB = seg(ab);
+    p.offParts = seg((size_t)batch * p.nparts * sizeof(float));
+    p.total = off;
+    return 0;
+}
+
+inline bf16_t* wsp(void* ws, size_t off) { return (bf16_t*)((char*)ws + off); }
+
+int check_ws(const void* ws) {
+    if (!ws) return fail(MUON_HIP_EINVAL, "workspace is null");
+    if (((uintptr_t)ws) & 255) return fail(MUON_HIP_EINVAL, "workspace must be 256-byte aligned");
+    return 0;
+}
+
+int check_gemm(int cfg, int Mp, int Kp, int batch, int& tile) {
+    tile = gemm_cfg_tile(cfg);
+    if (tile == 0) return fail(MUON_HIP_EINVAL, "unknown GEMM configuration %d", cfg);
+    if (Mp <= 0 || Kp <= 0 || batch <= 0) return fail(MUON_HIP_EINVAL, "sizes must be positive");
+    if (Mp % tile || Kp % tile) return fail(MUON_HIP_ESHAPE, "Mp=%d, Kp=%d must be multiples of the %d tile", Mp, Kp, tile);
+    const long T = Mp / tile, TN = Kp / tile;
+    if (T * TN * batch > 0x7fffffffL) return fail(MUON_HIP_ESHAPE, "too many tiles for one launch");
+    return 0;
+}
+
+int do_syrk(int cfg, const bf16_t* X, bf16_t* A, int Mp, int Kp, int batch, hipStream_t s) {
+    GemmArgs g = {};
+    const int tile = gemm_cfg_tile(cfg), T = Mp / tile;
+    g.P = g.Q = X;
+    g.strideP = g.strideQ = (long)Mp * Kp;
+    g.ldp = g.ldq = Kp;
+    g.kdim = Kp;
+    g.tiles_m = g.tiles_n = T;
+    g.tiles_per_mat = T * (T + 1) / 2;
+    g.batch = batch;
+    g.C = g.Ct = A;
+    g.strideC = g.strideCt = (long)Mp * Mp;
+    g.ldc = g.ldct = Mp;
+    Timed t(MUON_HIP_K_SYRK, s);
+    hipError_t e = launch_gemm_nt(cfg, EPI_SYRK, g, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "syrk launch");
+}
+
+int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b, double c, hipStream_t s) {
+    GemmArgs g = {};
+    const int tile = gemm_cfg_tile(cfg), T = Mp / tile;
+    g.P = g.Q = A;
+    g.strideP = g.strideQ = (long)Mp * Mp;
+    g.ldp = g.ldq = Mp;
+    g.kdim = Mp;
+    g.tiles_m = g.tiles_n = T;
+    g.tiles_per_mat = T * (T + 1) / 2;
+    g.batch = batch;
+    g.C = g.Ct = B;
+    g.strideC = g.strideCt = (long)Mp * Mp;
+    g.ldc = g.ldct = Mp;
+    g.Et = A;
+    g.strideEt = (long)Mp * Mp;
+    g.ldet = Mp;
+    g.s0 = (float)b;
+    g.s1 = (float)c;
+    Timed t(MUON_HIP_K_SYMPOLY, s);
+    hipError_t e = launch_gemm_nt(cfg, EPI_SYMPOLY, g, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "sympoly launch");
+}
+
+int do_bx(int cfg, const bf16_t* B, const bf16_t* XT, bf16_t* Xout, bf16_t* XTout, int Mp, int Kp, int batch,
+          double a, hipStream_t s) {
+    GemmArgs g = {};
+    const int tile = gemm_cfg_tile(cfg);
+    g.P = B;
+    g.strideP = (long)Mp * Mp;
+    g.ldp = Mp;
+    g.Q = XT;
+    g.strideQ = (long)Mp * Kp;
+    g.ldq = Mp;
+    g.kdim = Mp;
+    g.tiles_m = Mp / tile;
+    g.tiles_n = Kp / tile;
+    g.tiles_per_mat = g.tiles_m * g.tiles_n;
+    g.batch = batch;
+    g.C = Xout;
+    g.strideC = (long)Mp * Kp;
+    g.ldc = Kp;
+    g.Ct = XTout;
+    g.strideCt = (long)Mp * Kp;
+    g.ldct = Mp;
+    g.Et = XT;
+    g.strideEt = (long)Mp * Kp;
+    g.ldet = Mp;
+    g.s0 = (float)a;
+    Timed t(MUON_HIP_K_BX, s);
+    hipError_t e = launch_gemm_nt(cfg, EPI_BX, g, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "bx launch");
+}
+
+int dtype_ok(int d) { return d == MUON_HIP_F32 || d == MUON_HIP_BF16; }
+
+}  // namespace
+
+extern "C" {
+
+int muon_hip_version(void) { return 100; }
+
+const char* muon_hip_last_error(void) { return g_err; }
+
+int muon_hip_set_gemm_config(int cfg) {
+    if (cfg != MUON_HIP_CFG_AUTO && gemm_cfg_tile(cfg) == 0) return fail(MUON_HIP_EINVAL, "unknown GEMM configuration %d", cfg);
+    g_forced_cfg = cfg;
+    return 0;
+}
+
+int muon_hip_geometry(int rows, int cols, int* M, int* K, int* Mp, int* Kp, int* tile) {
+    Plan p;
+    if (int rc = make_plan(rows, cols, 1, p)) return rc;
+    if (M) *M = p.M;
+    if (K) *K = p.K;
+    if (Mp) *Mp = p.Mp;
+    if (Kp) *Kp = p.Kp;
+    if (tile) *tile = p.tile;
+    return 0;
+}
+
+size_t muon_hip_workspace_bytes(int rows, int cols, int batch) {
+    Plan p;
+    if (make_plan(rows, cols, batch, p)) return 0;
+    return p.total;
+}
+
+int muon_hip_momentum_norm(const void* const* g_ptrs, const void* const* m_ptrs, int g_dtype, int m_dtype,
+                           void* workspace, int rows, int cols, int batch, double beta, int nesterov,
+                           int write_back_grad, void* stream) {
+    Plan p;
+    if (int rc = make_plan(rows, cols, batch, p)) return rc;
+    if (int rc = check_ws(workspace)) return rc;
+    if (!g_ptrs || !m_ptrs) return fail(MUON_HIP_EINVAL, "pointer table is null");
+    const bool combo = (g_dtype == MUON_HIP_F32 && m_dtype == MUON_HIP_F32) ||
+                       (g_dtype == MUON_HIP_BF16 && (m_dtype == MUON_HIP_F32 || m_dtype == MUON_HIP_BF16));
+    if (!combo) return fail(MUON_HIP_EINVAL, "unsupported (grad, momentum) dtypes (%d, %d)", g_dtype, m_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_MOMENTUM, s);
+    hipError_t e = launch_momentum_norm(g_ptrs, m_ptrs, g_dtype, m_dtype, wsp(workspace, p.offX[1]), p.strideU,
+                                        (float*)((char*)workspace + p.offParts), p.nparts, p.n, batch, beta, nesterov,
+                                        write_back_grad, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "momentum_norm launch");
+}
+
+int muon_hip_cast_norm(const void* G, int g_dtype, void* workspace, int rows, int cols, int batch, void* stream) {
+    Plan p;
+    if (int rc = make_plan(rows, cols, batch, p)) return rc;
+    if (int rc = check_ws(workspace)) return rc;
+    if (!G || !dtype_ok(g_dtype)) return fail(MUON_HIP_EINVAL, "bad input tensor or dtype");
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_MOMENTUM, s);
+    hipError_t e = launch_cast_norm(G, p.n, g_dtype, wsp(workspace, p.offX[1]), p.strideU,
+                                    (float*)((char*)workspace + p.offParts), p.nparts, p.n, batch, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "cast_norm launch");
+}
+
+int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int steps, double a, double b, double c,
+                        void* stream) {
+    Plan p;
+    if (int rc = make_plan(rows, cols, batch, p)) return rc;
+    if (int rc = check_ws(workspace)) return rc;
+    if (steps < 0) return fail(MUON_HIP_EINVAL, "steps must be >= 0");
+    hipStream_t s = (hipStream_t)stream;
+    bf16_t* X[2] = {wsp(workspace, p.offX[0]), wsp(workspace, p.offX[1])};
+    bf16_t* XT[2] = {wsp(workspace, p.offXT[0]), wsp(workspace, p.offXT[1])};
+    bf16_t* A = wsp(workspace, p.offA);
+    bf16_t* B = wsp(workspace, p.offB);
+    {
+        Timed t(MUON_HIP_K_NORMALIZE, s);
+        hipError_t e = launch_normalize(X[1], p.strideU, (const float*)((char*)workspace + p.offParts), p.nparts, X[0],
+                                        XT[0], p.strideX, rows, cols, p.Mp, p.Kp, batch, s);
+        if (e != hipSuccess) return hip_fail(e, "normalize launch");
+    }
+    int cur = 0;
+    for (int it = 0; it < steps; ++it) {
+        const bool last = it + 1 == steps;
+        if (int rc = do_syrk(p.cfg, X[cur], A, p.Mp, p.Kp, batch, s)) return rc;
+        if (int rc = do_sympoly(p.cfg, A, B, p.Mp, batch, b, c, s)) return rc;
+        bf16_t* xo = (last && p.transposed) ? nullptr : X[cur ^ 1];
+        bf16_t* xto = (last && !p.transposed) ? nullptr : XT[cur ^ 1];
+        if (int rc = do_bx(p.cfg, B, XT[cur], xo, xto, p.Mp, p.Kp, batch, a, s)) return rc;
+        cur ^= 1;
+    }
+    return 0;
+}
+
+int muon_hip_apply_update(const void* const* p_ptrs, int p_dtype, void* workspace, int rows, int cols, int batch,
+                          int steps, double scale, double lr, double weight_decay, void* stream) {
+    Plan p;
+    if (int rc = make_plan(rows, cols, batch, p)) return rc;
+    if (int rc = check_ws(workspace)) return rc;
+    if (!p_ptrs || !dtype_ok(p_dtype) || steps < 0) return fail(MUON_HIP_EINVAL, "bad pointer table, dtype or steps");
+    hipStream_t s = (hipStream_t)stream;
+    const int cur = steps & 1;
+    const bf16_t* O = wsp(workspace, p.transposed ? p.offXT[cur] : p.offX[cur]);
+    const int ldo = p.transposed ? p.Mp : p.Kp;
+    Timed t(MUON_HIP_K_UPDATE, s);
+    hipError_t e = launch_apply_update(p_ptrs, p_dtype, O, p.strideX, ldo, rows, cols, batch, scale, lr, weight_decay, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "apply_update launch");
+}
+
+int muon_hip_ns_output(void* workspace, int rows, int cols, int batch, int steps, void* out, void* stream) {
+    Plan p;
+    if (int rc = make_plan(rows, cols, batch, p)) return rc;
+    if (int rc = check_ws(workspace)) return rc;
+    if (!out || steps < 0) return fail(MUON_HIP_EINVAL, "bad output pointer or steps");
+    hipStream_t s = (hipStream_t)stream;
+    const int cur = steps & 1;
+    const bf16_t* O = wsp(workspace, p.transposed ? p.offXT[cur] : p.offX[cur]);
+    const int ldo = p.transposed ? p.Mp : p.Kp;
+    hipError_t e = launch_gather_output((bf16_t*)out, p.n, O, p.strideX, ldo, rows, cols, batch, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "ns_output launch");
+}
+
+int muon_hip_step_grouped(const void* const* p_ptrs, const void* const* g_ptrs, const void* const* m_ptrs,
+                          int p_dtype, int g_dtype, int m_dtype, void* workspace, int rows, int cols, int batch,
+                          double lr, double weight_decay, double beta, int nesterov, int ns_steps, double scale,
+                          double a, double b, double c, int write_back_grad, void* stream) {
+    if (int rc = muon_hip_momentum_norm(g_ptrs, m_ptrs, g_dtype, m_dtype, workspace, rows, cols, batch, beta, nesterov,
+                                        write_back_grad, stream))
+        return rc;
+    if (int rc = muon_hip_ns_grouped(workspace, rows, cols, batch, ns_steps, a, b, c, stream)) return rc;
+    return muon_hip_apply_update(p_ptrs, p_dtype, workspace, rows, cols, batch, ns_steps, scale, lr, weight_decay,
+                                 stream);
+}
+
+int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* stream) {
+    if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp);
+    int tile;
+    if (int rc = check_gemm(cfg, Mp, Kp, batch, tile)) return rc;
+    if (!X || !A) return fail(MUON_HIP_EINVAL, "null operand");
+    return do_syrk(cfg, (const bf16_t*)X, (bf16_t*)A, Mp, Kp, batch, (hipStream_t)stream);
+}
+
+int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* stream) {
+    if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp);
+    int tile;
+    if (int rc = check_gemm(cfg, Mp, Mp, batch, tile)) return rc;
+    if (!A || !B || A == B) return fail(MUON_HIP_EINVAL, "null or aliased operand");
+    return do_sympoly(cfg, (const bf16_t*)A, (bf16_t*)B, Mp, batch, b, c, (hipStream_t)stream);
+}
+
+int muon_hip_bx_axpy_bf16(const void* B, const void* XT, void* Xout, void* XTout, int Mp, int Kp, int batch,
+                          double a, int cfg, void* stream) {
+    if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp);
+    int tile;
+    if (int rc = check_gemm(cfg, Mp, Kp, batch, tile)) return rc;
+    if (!B || !XT || (!Xout && !XTout)) return fail(MUON_HIP_EINVAL, "null operand");
+    if (XTout == XT) return fail(MUON_HIP_EINVAL, "XTout must not alias XT");
+    return do_bx(cfg, (const bf16_t*)B, (const bf16_t*)XT, (bf16_t*)Xout, (bf16_t*)XTout, Mp, Kp, batch, a,
+                 (hipStream_t)stream);
+}
+
+int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int dtype, long n, int step, double lr,
+                   double beta1, double beta2, double eps, double weight_decay, void* stream) {
+    if (!p || !g || !exp_avg || !exp_avg_sq) return fail(MUON_HIP_EINVAL, "null tensor");
+    if (!dtype_ok(dtype) || n < 0 || step < 1) return fail(MUON_HIP_EINVAL, "bad dtype, size or step");
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_ADAMW, s);
+    hipError_t e = launch_adamw(p, g, exp_avg, exp_avg_sq, dtype, n, step, lr, beta1, beta2, eps, weight_decay, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "adamw launch");
+}
+
+int muon_hip_timing_enable(int on) {
+    std::lock_guard<std::mutex> lk(g_tmu);
+    clear_events();
+    g_timing = on != 0;
+    return 0;
+}
+
+int muon_hip_timing_read(int kernel_id, double* total_ms, long* launches) {
+    if (kernel_id < 0 || kernel_id >= MUON_HIP_K_COUNT || !total_ms || !launches)
+        return fail(MUON_HIP_EINVAL, "bad kernel id or null output");
+    std::lock_guard<std::mutex> lk(g_tmu);
+    double tot = 0.0;
+    for (auto& p : g_events[kernel_id]) {
+        hipError_t e = hipEventSynchronize(p.stop);
+        if (e != hipSuccess) return hip_fail(e, "event synchronize");
+        float ms = 0.f;
+        e = hipEventElapsedTime(&ms, p.start, p.stop);
+        if (e != hipSuccess) return hip_fail(e, "event elapsed");
+        tot += ms;
+    }
+    *total_ms = tot;
+    *launches = (long)g_events[kernel_id].size();
+    return 0;
+}
+
+}  // extern "C"

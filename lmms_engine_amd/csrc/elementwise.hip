@@ -1,0 +1,390 @@
+// HBM-bound kernels of the Muon step on gfx950: momentum/Nesterov blend with Frobenius
+// partial sums, normalisation into the two padded operand layouts, the scaled parameter
+// update, and the AdamW fallback.  128-bit accesses on the aligned path, a scalar path
+// otherwise.  All reductions are two-stage with a fixed order, so results are
+// run-to-run bit identical (no float atomics).
+//
+// Arithmetic follows /root/reference/src/lmms_engine/utils/muon_utils.py:
+//   momentum_norm : muon_update's lerp_ pair (:188-189) + X = G.bfloat16() (:138) + the
+//                   sum of squares feeding X.norm (:146)
+//   normalize     : X / (X.norm + 1e-7) (:146) and the rows>cols transpose (:139-140)
+//   apply_update  : apply_scaling (:167-175) + param.mul_/add_ (:324-325)
+//   adamw         : adam_update (:178-183) + the Adam branch (:468-477)
+#include "common.h"
+#include "elementwise.h"
+
+namespace {
+
+template <typename T> struct Ld;
+template <> struct Ld<float> {
+    static __device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+        const f32x4 a = *(const f32x4*)p, b = *(const f32x4*)(p + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+    }
+    static __device__ __forceinline__ void store8(float* p, const float (&v)[8]) {
+        f32x4 a, b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { a[i] = v[i]; b[i] = v[4 + i]; }
+        *(f32x4*)p = a;
+        *(f32x4*)(p + 4) = b;
+    }
+    static __device__ __forceinline__ float rnd(float x) { return x; }
+    static __device__ __forceinline__ float load(const float* p) { return *p; }
+    static __device__ __forceinline__ void store(float* p, float x) { *p = x; }
+};
+template <> struct Ld<bf16_t> {
+    static __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+        const bf16x8 a = *(const bf16x8*)p;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = bf2f(a[i]);
+    }
+    static __device__ __forceinline__ void store8(bf16_t* p, const float (&v)[8]) {
+        bf16x8 a;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] = f2bf(v[i]);
+        *(bf16x8*)p = a;
+    }
+    static __device__ __forceinline__ float rnd(float x) { return rbf(x); }
+    static __device__ __forceinline__ float load(const bf16_t* p) { return bf2f(*p); }
+    static __device__ __forceinline__ void store(bf16_t* p, float x) { *p = f2bf(x); }
+};
+
+// ATen's lerp with a scalar weight, one fma: |w| < 0.5 -> s + w (e - s), else
+// e - (e - s)(1 - w).  wm1 = w - 1 (exact in fp32 for w in [0.5, 2]).
+__device__ __forceinline__ float lerp_aten(float s, float e, float w, float wm1, bool small) {
+    const float d = e - s;
+    return small ? fmaf(w, d, s) : fmaf(wm1, d, e);
+}
+
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+struct MomentumMath {
+    float w1, w1m1, w2, w2m1;
+    bool small1, small2, nesterov;
+};
+
+template <typename GT, typename MT>
+__device__ __forceinline__ float momentum_one(float g, float m, const MomentumMath& mm, float& m_out) {
+    const float mn = Ld<MT>::rnd(lerp_aten(m, g, mm.w1, mm.w1m1, mm.small1));
+    m_out = mn;
+    return mm.nesterov ? lerp_aten(g, mn, mm.w2, mm.w2m1, mm.small2) : mn;
+}
+
+template <typename GT, typename MT>
+__global__ void __launch_bounds__(256)
+momentum_norm_kernel(const void* const* g_ptrs, const void* const* m_ptrs, bf16_t* U, long strideU,
+                     float* partials, long n, MomentumMath mm, int write_back) {
+    __shared__ float red[4];
+    const int b = blockIdx.y;
+    GT* g = (GT*)g_ptrs[b];
+    MT* m = (MT*)m_ptrs[b];
+    bf16_t* u = U + b * strideU;
+    float ss = 0.f;
+    const bool vec = ((((uintptr_t)g) | ((uintptr_t)m)) & 15) == 0;
+    const long n8 = vec ? n / 8 : 0;
+    for (long i8 = (long)blockIdx.x * 256 + threadIdx.x; i8 < n8; i8 += (long)gridDim.x * 256) {
+        float gv[8], mv[8], uv[8];
+        Ld<GT>::load8(g + i8 * 8, gv);
+        Ld<MT>::load8(m + i8 * 8, mv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float mo;
+            float uu = momentum_one<GT, MT>(gv[i], mv[i], mm, mo);
+            mv[i] = mo;
+            if (write_back) gv[i] = uu;
+            uu = rbf(uu);
+            uv[i] = uu;
+            ss = fmaf(uu, uu, ss);
+        }
+        Ld<MT>::store8(m + i8 * 8, mv);
+        Ld<bf16_t>::store8(u + i8 * 8, uv);
+        if (write_back) Ld<GT>::store8(g + i8 * 8, gv);
+    }
+    // scalar tail (or everything when the pointers are not 16-byte aligned)
+    for (long i = n8 * 8 + (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        float mo;
+        float uu = momentum_one<GT, MT>(Ld<GT>::load(g + i), Ld<MT>::load(m + i), mm, mo);
+        Ld<MT>::store(m + i, mo);
+        if (write_back) Ld<GT>::store(g + i, uu);
+        uu = rbf(uu);
+        u[i] = f2bf(uu);
+        ss = fmaf(uu, uu, ss);
+    }
+    ss = block_sum_256(ss, red);
+    if (threadIdx.x == 0) partials[(long)b * gridDim.x + blockIdx.x] = ss;
+}
+
+// Sum of squares of an existing bf16 (or fp32, rounded to bf16 first) matrix: the
+// Frobenius stage of fast_newtonschulz when it is called on its own.
+template <typename GT>
+__global__ void __launch_bounds__(256)
+cast_norm_kernel(const GT* G, long strideG, bf16_t* U, long strideU, float* partials, long n) {
+    __shared__ float red[4];
+    const int b = blockIdx.y;
+    const GT* g = G + b * strideG;
+    bf16_t* u = U + b * strideU;
+    float ss = 0.f;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        const float uu = rbf(Ld<GT>::load(g + i));
+        u[i] = f2bf(uu);
+        ss = fmaf(uu, uu, ss);
+    }
+    ss = block_sum_256(ss, red);
+    if (threadIdx.x == 0) partials[(long)b * gridDim.x + blockIdx.x] = ss;
+}
+
+// d = bf(bf(sqrt(sum)) + 1e-7), the same value in every block of a matrix.
+__device__ __forceinline__ float frob_denominator(const float* part, int nparts, float* red) {
+    float s = 0.f;
+    for (int i = threadIdx.x; i < nparts; i += 256) s += part[i];
+    s = block_sum_256(s, red);
+    const float nrm = rbf(__fsqrt_rn(s));
+    return rbf(nrm + 1e-7f);
+}
+
+// One 64x64 tile of the padded operand X (Mp x Kp) and of its transposed copy Xt (Kp x Mp)
+// from the bf16 blend u held in the parameter's own layout (rows x cols).
+__global__ void __launch_bounds__(256)
+normalize_kernel(const bf16_t* U, long strideU, const float* partials, int nparts, bf16_t* X, bf16_t* XT,
+                 long strideX, int rows, int cols, int Mp, int Kp) {
+    __shared__ float red[4];
+    __shared__ __align__(16) bf16_t tile[64][72];
+    const int b = blockIdx.y;
+    const float d = frob_denominator(partials + (long)b * nparts, nparts, red);
+    const bf16_t* u = U + b * strideU;
+    // The tile is addressed in the parameter's orientation: r over rows, c over cols.
+    // transposed (rows > cols): X = u^T, so the padded row-major image of u is Xt.
+    const bool transposed = rows > cols;
+    const int Rp = transposed ? Kp : Mp, Cp = transposed ? Mp : Kp;  // padded rows/cols of u's image
+    bf16_t* same = (transposed ? XT : X) + b * strideX;               // same orientation as u
+    bf16_t* flip = (transposed ? X : XT) + b * strideX;               // the transposed image
+    const int tiles_c = Cp / 64;
+    const int r0 = (blockIdx.x / tiles_c) * 64, c0 = (blockIdx.x % tiles_c) * 64;
+    const int tr = threadIdx.x >> 3, tc = (threadIdx.x & 7) * 8;
+    const bool vec = (cols % 8) == 0;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int r = r0 + tr + h * 32, c = c0 + tc;
+        bf16x8 o;
+        if (r < rows && vec && c + 8 <= cols) {
+            const bf16x8 v = *(const bf16x8*)(u + (long)r * cols + c);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) o[i] = f2bf(__fdiv_rn(bf2f(v[i]), d));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float x = 0.f;
+                if (r < rows && c + i < cols) x = __fdiv_rn(bf2f(u[(long)r * cols + c + i]), d);
+                o[i] = f2bf(x);
+            }
+        }
+        *(bf16x8*)(&tile[tr + h * 32][tc]) = o;
+        *(bf16x8*)(same + (long)r * Cp + c) = o;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        // flip[c][r]: row index over cols, 8 consecutive r per thread
+        const int fc = tr + h * 32, fr = tc;
+        bf16x8 o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = tile[fr + i][fc];
+        *(bf16x8*)(flip + (long)(c0 + fc) * Rp + r0 + fr) = o;
+    }
+}
+
+struct UpdateMath {
+    float scale, decay, alpha;
+};
+
+template <typename PT>
+__device__ __forceinline__ float update_one(float p, float o, const UpdateMath& um) {
+    const float os = rbf(o * um.scale);
+    const float pd = Ld<PT>::rnd(p * um.decay);
+    return fmaf(um.alpha, os, pd);
+}
+
+// p <- p (1 - lr wd) - lr bf(O s); O is the NS output in the parameter's orientation with
+// a padded row stride.
+template <typename PT>
+__global__ void __launch_bounds__(256)
+apply_update_kernel(const void* const* p_ptrs, const bf16_t* O, long strideO, int ldo, int rows, int cols,
+                    UpdateMath um) {
+    const int b = blockIdx.y;
+    PT* p = (PT*)p_ptrs[b];
+    const bf16_t* o = O + b * strideO;
+    const bool vec = (cols % 8 == 0) && ((((uintptr_t)p) & 15) == 0);
+    if (vec) {
+        const int gpr = cols / 8;
+        const long n8 = (long)rows * gpr;
+        for (long i8 = (long)blockIdx.x * 256 + threadIdx.x; i8 < n8; i8 += (long)gridDim.x * 256) {
+            const long r = i8 / gpr;
+            const int c = (int)(i8 - r * gpr) * 8;
+            float pv[8], ov[8];
+            Ld<PT>::load8(p + i8 * 8, pv);
+            Ld<bf16_t>::load8(o + r * ldo + c, ov);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pv[i] = update_one<PT>(pv[i], ov[i], um);
+            Ld<PT>::store8(p + i8 * 8, pv);
+        }
+    } else {
+        const long n = (long)rows * cols;
+        for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+            const long r = i / cols;
+            const int c = (int)(i - r * cols);
+            Ld<PT>::store(p + i, update_one<PT>(Ld<PT>::load(p + i), bf2f(o[r * ldo + c]), um));
+        }
+    }
+}
+
+// Scaled NS output into a dense (rows x cols) bf16 tensor: fast_newtonschulz called alone.
+__global__ void __launch_bounds__(256)
+gather_output_kernel(bf16_t* out, long strideOut, const bf16_t* O, long strideO, int ldo, int rows, int cols) {
+    const int b = blockIdx.y;
+    const long n = (long)rows * cols;
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        const long r = i / cols;
+        const int c = (int)(i - r * cols);
+        out[b * strideOut + i] = O[b * strideO + r * ldo + c];
+    }
+}
+
+struct AdamMath {
+    float w1, w1m1, w2, w2m1, c1, c2, eps, decay, alpha;
+    bool small1, small2;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+adamw_kernel(T* p, const T* g, T* e1, T* e2, long n, AdamMath am) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        const float gi = Ld<T>::load(g + i);
+        const float a = Ld<T>::rnd(lerp_aten(Ld<T>::load(e1 + i), gi, am.w1, am.w1m1, am.small1));
+        const float g2 = Ld<T>::rnd(gi * gi);
+        const float bb = Ld<T>::rnd(lerp_aten(Ld<T>::load(e2 + i), g2, am.w2, am.w2m1, am.small2));
+        Ld<T>::store(e1 + i, a);
+        Ld<T>::store(e2 + i, bb);
+        const float ac = Ld<T>::rnd(__fdiv_rn(a, am.c1));
+        const float bc = Ld<T>::rnd(__fdiv_rn(bb, am.c2));
+        const float den = Ld<T>::rnd(Ld<T>::rnd(__fsqrt_rn(bc)) + am.eps);
+        const float upd = Ld<T>::rnd(__fdiv_rn(ac, den));
+        const float pd = Ld<T>::rnd(Ld<T>::load(p + i) * am.decay);
+        Ld<T>::store(p + i, fmaf(am.alpha, upd, pd));
+    }
+}
+
+inline int blocks_for(long n, int per_block, int cap) {
+    long b = (n + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    if (b > cap) b = cap;
+    return (int)b;
+}
+
+inline void lerp_consts(double weight, float& w, float& wm1, bool& small) {
+    w = (float)weight;
+    wm1 = w - 1.0f;
+    small = fabsf(w) < 0.5f;
+}
+
+}  // namespace
+
+int momentum_parts(long n) { return blocks_for(n, 256 * 8 * 4, MUON_MAX_PARTS); }
+
+hipError_t launch_momentum_norm(const void* const* g_ptrs, const void* const* m_ptrs, int g_dtype, int m_dtype,
+                                bf16_t* U, long strideU, float* partials, int nparts, long n, int batch,
+                                double beta, int nesterov, int write_back, hipStream_t stream) {
+    MomentumMath mm;
+    lerp_consts(1.0 - beta, mm.w1, mm.w1m1, mm.small1);
+    lerp_consts(beta, mm.w2, mm.w2m1, mm.small2);
+    mm.nesterov = nesterov != 0;
+    dim3 grid(nparts, batch), block(256);
+    if (g_dtype == MUON_HIP_F32 && m_dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((momentum_norm_kernel<float, float>), grid, block, 0, stream, g_ptrs, m_ptrs, U, strideU,
+                           partials, n, mm, write_back);
+    else if (g_dtype == MUON_HIP_BF16 && m_dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((momentum_norm_kernel<bf16_t, float>), grid, block, 0, stream, g_ptrs, m_ptrs, U, strideU,
+                           partials, n, mm, write_back);
+    else if (g_dtype == MUON_HIP_BF16 && m_dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((momentum_norm_kernel<bf16_t, bf16_t>), grid, block, 0, stream, g_ptrs, m_ptrs, U, strideU,
+                           partials, n, mm, write_back);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_cast_norm(const void* G, long strideG, int g_dtype, bf16_t* U, long strideU, float* partials,
+                            int nparts, long n, int batch, hipStream_t stream) {
+    dim3 grid(nparts, batch), block(256);
+    if (g_dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((cast_norm_kernel<float>), grid, block, 0, stream, (const float*)G, strideG, U, strideU,
+                           partials, n);
+    else if (g_dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((cast_norm_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)G, strideG, U, strideU,
+                           partials, n);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, bf16_t* X, bf16_t* XT,
+                            long strideX, int rows, int cols, int Mp, int Kp, int batch, hipStream_t stream) {
+    dim3 grid((Mp / 64) * (Kp / 64), batch), block(256);
+    hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, partials, nparts, X, XT, strideX, rows,
+                       cols, Mp, Kp);
+    return hipGetLastError();
+}
+
+hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf16_t* O, long strideO, int ldo,
+                               int rows, int cols, int batch, double scale, double lr, double wd,
+                               hipStream_t stream) {
+    UpdateMath um;
+    um.scale = (float)scale;
+    um.decay = (float)(1.0 - lr * wd);
+    um.alpha = (float)(-lr);
+    dim3 grid(blocks_for((long)rows * cols, 256 * 8 * 4, 2048), batch), block(256);
+    if (p_dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((apply_update_kernel<float>), grid, block, 0, stream, p_ptrs, O, strideO, ldo, rows, cols, um);
+    else if (p_dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((apply_update_kernel<bf16_t>), grid, block, 0, stream, p_ptrs, O, strideO, ldo, rows, cols,
+                           um);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_gather_output(bf16_t* out, long strideOut, const bf16_t* O, long strideO, int ldo, int rows,
+                                int cols, int batch, hipStream_t stream) {
+    dim3 grid(blocks_for((long)rows * cols, 256 * 8, 2048), batch), block(256);
+    hipLaunchKernelGGL(gather_output_kernel, grid, block, 0, stream, out, strideOut, O, strideO, ldo, rows, cols);
+    return hipGetLastError();
+}
+
+hipError_t launch_adamw(void* p, const void* g, void* e1, void* e2, int dtype, long n, int step, double lr,
+                        double b1, double b2, double eps, double wd, hipStream_t stream) {
+    AdamMath am;
+    lerp_consts(1.0 - b1, am.w1, am.w1m1, am.small1);
+    lerp_consts(1.0 - b2, am.w2, am.w2m1, am.small2);
+    am.c1 = (float)(1.0 - pow(b1, (double)step));
+    am.c2 = (float)(1.0 - pow(b2, (double)step));
+    am.eps = (float)eps;
+    am.decay = (float)(1.0 - lr * wd);
+    am.alpha = (float)(-lr);
+    dim3 grid(blocks_for(n, 256 * 4, 8192)), block(256);
+    if (dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((adamw_kernel<float>), grid, block, 0, stream, (float*)p, (const float*)g, (float*)e1,
+                           (float*)e2, n, am);
+    else if (dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((adamw_kernel<bf16_t>), grid, block, 0, stream, (bf16_t*)p, (const bf16_t*)g, (bf16_t*)e1,
+                           (bf16_t*)e2, n, am);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}

@@ -1,0 +1,31 @@
+// Host-side description of one batched NT GEMM launch (see gemm_nt.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include "common.h"
+
+enum { EPI_SYRK = 0, EPI_SYMPOLY = 1, EPI_BX = 2 };
+enum { GEMM_CFG_128x128_W4 = 0, GEMM_CFG_256x256_W4 = 1, GEMM_CFG_256x256_W8 = 2, GEMM_CFG_COUNT = 3 };
+
+struct GemmArgs {
+    const bf16_t* P;   // left operand rows (reduction contiguous)
+    const bf16_t* Q;   // right operand rows (reduction contiguous)
+    long strideP, strideQ;  // elements between matrices of the batch
+    int ldp, ldq;           // elements between rows
+    int kdim;               // reduction length, a multiple of 64
+    int tiles_m, tiles_n;   // tile grid of one matrix (triangular kernels: tiles_m == tiles_n)
+    int tiles_per_mat;      // tiles_m*(tiles_m+1)/2 for the symmetric kernels, tiles_m*tiles_n for BX
+    int batch;
+    bf16_t* C;    // out[i][j]; may be null for BX
+    long strideC;
+    int ldc;
+    bf16_t* Ct;   // out[j][i]; the same buffer as C for the symmetric kernels; may be null for BX
+    long strideCt;
+    int ldct;
+    const bf16_t* Et;  // elementwise source read as Et[j][i]: A (symmetric) or Xt
+    long strideEt;
+    int ldet;
+    float s0, s1;  // SYMPOLY: (b, c); BX: (a, -)
+};
+
+int gemm_cfg_tile(int cfg);
+hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t stream);

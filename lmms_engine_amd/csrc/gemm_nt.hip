@@ -1,0 +1,244 @@
+// NT GEMM family for the Newton-Schulz chain on gfx950 (v_mfma_f32_32x32x16_bf16).
+//
+// All three products of one NS iteration are "row times row" contractions of bf16
+// operands whose reduction dimension is contiguous:
+//   SYRK     A  = bf(X Xt)                         P = Q = X   (M x K)
+//   SYMPOLY  B  = bf(bf(b A) + bf(c bf(A A)))      P = Q = A   (M x M, symmetric so A A = A At)
+//   BX       X' = bf(bf(a X) + bf(B X))            P = B (M x M), Q = Xt (K x M)
+// BX reads the transposed copy Xt as its second operand and writes both X' and X't, so no
+// operand ever needs a transposing load.  SYRK/SYMPOLY compute only tiles on or above the
+// diagonal and mirror them, which makes the result symmetric bit for bit.
+//
+// Every bf16 rounding point of the reference's torch expressions
+// (/root/reference/src/lmms_engine/utils/muon_utils.py:149-152) is applied in registers.
+//
+// Operands are zero padded by the caller to whole tiles, so there is no masking here; the
+// host launcher checks that the shapes it is given are whole tiles before launching.
+#include "common.h"
+#include "gemm_nt.h"
+
+namespace {
+
+constexpr int BK = 64;          // bf16 elements per k-tile: one 128-byte LDS row
+constexpr int ROW_BYTES = 128;
+
+// Upper-triangle tile order in row groups of GM: inside a group, column by column, so the
+// ~32 tiles an XCD works on at a time touch few distinct row panels.
+template <int GM>
+__device__ __forceinline__ void tri_decode(int t, int T, int& ti, int& tj) {
+    int r0 = 0;
+    for (;;) {
+        const int gm = (T - r0 < GM) ? (T - r0) : GM;
+        const int cnt = gm * (T - r0) - gm * (gm - 1) / 2;
+        if (t < cnt || r0 + gm >= T) {
+            const int tri = gm * (gm + 1) / 2;
+            if (t < tri) {
+                int c = 0;  // column c of the leading gm x gm triangle holds c+1 tiles
+                while (t >= c + 1) { t -= c + 1; ++c; }
+                ti = r0 + t;
+                tj = r0 + c;
+            } else {
+                t -= tri;
+                tj = r0 + gm + t / gm;
+                ti = r0 + t % gm;
+            }
+            return;
+        }
+        t -= cnt;
+        r0 += gm;
+    }
+}
+
+template <int GM>
+__device__ __forceinline__ void rect_decode(int t, int TM, int TN, int& ti, int& tj) {
+    const int per_group = GM * TN;
+    const int gidx = t / per_group;
+    const int first = gidx * GM;
+    const int gm = (TM - first < GM) ? (TM - first) : GM;
+    const int r = t - gidx * per_group;
+    ti = first + r % gm;
+    tj = r / gm;
+}
+
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE = A_BYTES + B_BYTES;
+    constexpr int CA = BM * 8 / NT, CB = BN * 8 / NT;  // 16-byte chunks per thread per k-tile
+    constexpr int RSTEP = NT / 8;                      // rows between a thread's chunks
+    static_assert(BM % (WGM * 32) == 0 && BN % (WGN * 32) == 0, "wave tiling");
+    static_assert((BM * 8) % NT == 0 && (BN * 8) % NT == 0 && RSTEP % 16 == 0, "staging");
+    static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    const int bidx = logical / g.tiles_per_mat;
+    const int t = logical - bidx * g.tiles_per_mat;
+    int ti, tj;
+    if (EPI == EPI_BX) rect_decode<4>(t, g.tiles_m, g.tiles_n, ti, tj);
+    else tri_decode<4>(t, g.tiles_m, ti, tj);
+
+    const long m0 = (long)ti * BM, n0 = (long)tj * BN;
+    const bf16_t* Pb = g.P + bidx * g.strideP + m0 * g.ldp;
+    const bf16_t* Qb = g.Q + bidx * g.strideQ + n0 * g.ldq;
+
+    // ---- global -> register -> LDS staging -------------------------------------------
+    const int lrow = tid >> 3, lc = tid & 7;
+    const bf16_t* pa = Pb + (long)lrow * g.ldp + lc * 8;
+    const bf16_t* pb = Qb + (long)lrow * g.ldq + lc * 8;
+    // 16-byte chunk c of row r lives at r*128 + ((c ^ ((r>>1)&7)) << 4): the 16 rows one
+    // ds_read_b128 phase touches then cover all 64 banks once.
+    const int lds_w = lrow * ROW_BYTES + ((lc ^ ((lrow >> 1) & 7)) << 4);
+    u32x4 ra[CA], rb[CB];
+
+    auto gload = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < CA; ++i) ra[i] = *(const u32x4*)(pa + (long)i * RSTEP * g.ldp + k0);
+#pragma unroll
+        for (int i = 0; i < CB; ++i) rb[i] = *(const u32x4*)(pb + (long)i * RSTEP * g.ldq + k0);
+    };
+    auto lstore = [&](int stage) {
+        unsigned char* s = smem + stage * STAGE + lds_w;
+#pragma unroll
+        for (int i = 0; i < CA; ++i) *(u32x4*)(s + i * RSTEP * ROW_BYTES) = ra[i];
+#pragma unroll
+        for (int i = 0; i < CB; ++i) *(u32x4*)(s + A_BYTES + i * RSTEP * ROW_BYTES) = rb[i];
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int sw = (lane >> 1) & 7, hi = lane >> 5;
+    const int a_off = (wm * WTM + (lane & 31)) * ROW_BYTES;
+    const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROW_BYTES;
+
+    const int nk = g.kdim / BK;
+    gload(0);
+    lstore(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const bool more = kt + 1 < nk;
+        if (more) gload((kt + 1) * BK);
+        const unsigned char* st = smem + (kt & 1) * STAGE;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            const int co = (((ks << 1) | hi) ^ sw) << 4;
+            bf16x8 af[FM], bq[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) af[i] = *(const bf16x8*)(st + a_off + i * 32 * ROW_BYTES + co);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) bq[j] = *(const bf16x8*)(st + b_off + j * 32 * ROW_BYTES + co);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bq[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) lstore((kt + 1) & 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue ---------------------------------------------------------------------
+    // Lane (lane&31) owns column j; registers 4q..4q+3 are rows 8q + 4*(lane>>5) + 0..3.
+    const bool diag = (EPI != EPI_BX) && (ti == tj);
+    bf16_t* C = g.C ? g.C + bidx * g.strideC : nullptr;
+    bf16_t* Ct = g.Ct ? g.Ct + bidx * g.strideCt : nullptr;
+    const bf16_t* Et = g.Et ? g.Et + bidx * g.strideEt : nullptr;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const long gj = n0 + wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const long gi = m0 + wm * WTM + i * 32 + q * 8 + hi * 4;
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = rbf(acc[i][j][q * 4 + r]);
+                if (EPI != EPI_SYRK) {
+                    const bf16x4 e = *(const bf16x4*)(Et + gj * g.ldet + gi);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (EPI == EPI_SYMPOLY) v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + rbf(g.s1 * v[r]));
+                        else v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + v[r]);
+                    }
+                }
+                bf16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = f2bf(v[r]);
+                if (diag) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (gi + r <= gj) {
+                            C[(gi + r) * g.ldc + gj] = o[r];
+                            C[gj * g.ldc + gi + r] = o[r];
+                        }
+                    }
+                } else {
+                    if (C) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) C[(gi + r) * g.ldc + gj] = o[r];
+                    }
+                    if (Ct) *(bf16x4*)(Ct + gj * g.ldct + gi) = o;
+                }
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN, int EPI>
+hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
+    constexpr int smem = 2 * (BM + BN) * ROW_BYTES;
+    static bool configured = false;  // per instantiation; the attribute is idempotent
+    auto kern = gemm_nt_kernel<BM, BN, WGM, WGN, EPI>;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(nblocks), dim3(WGM * WGN * 64), smem, stream, g);
+    return hipGetLastError();
+}
+
+template <int EPI>
+hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t stream) {
+    switch (cfg) {
+        case GEMM_CFG_128x128_W4: return launch_one<128, 128, 2, 2, EPI>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W4: return launch_one<256, 256, 2, 2, EPI>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8: return launch_one<256, 256, 2, 4, EPI>(g, nblocks, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+int gemm_cfg_tile(int cfg) {
+    switch (cfg) {
+        case GEMM_CFG_128x128_W4: return 128;
+        case GEMM_CFG_256x256_W4:
+        case GEMM_CFG_256x256_W8: return 256;
+        default: return 0;
+    }
+}
+
+hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t stream) {
+    const int nblocks = g.tiles_per_mat * g.batch;
+    if (nblocks <= 0) return hipSuccess;
+    switch (epi) {
+        case EPI_SYRK: return launch_cfg<EPI_SYRK>(cfg, g, nblocks, stream);
+        case EPI_SYMPOLY: return launch_cfg<EPI_SYMPOLY>(cfg, g, nblocks, stream);
+        case EPI_BX: return launch_cfg<EPI_BX>(cfg, g, nblocks, stream);
+        default: return hipErrorInvalidValue;
+    }
+}

@@ -1,0 +1,435 @@
+"""Muon optimizer step on one MI355X: the host side.
+
+Mirrors the public surface of the reference module
+/root/reference/src/lmms_engine/utils/muon_utils.py (same names, argument meaning, group
+and state layout, error behaviour) so that `from ... import Muon` can be pointed here and
+the trainer's optimizer factory (src/lmms_engine/train/hf/trainer.py:459-465) works unchanged.
+All arithmetic runs in hand-written gfx950 kernels behind the C ABI of libmuon_hip.so
+(include/muon_hip.h); torch supplies device memory and streams only.  There is no
+fallback: tensors that are not on a GPU, or a missing library, raise.
+
+Differences from the reference, all deliberate:
+  * step() dispatches each stage once per bucket of same-shape parameters (pointer tables,
+    batched kernels) instead of once per parameter.
+  * keyword-correct hyper-parameters: `ns_steps` iterations and the `nesterov` flag mean what
+    they say.  The reference's single-device call site passes them swapped positionally
+    (muon_utils.py:316-323 into :186); `reference_bug_compat=True` reproduces that.
+  * p.grad is not overwritten with the Nesterov blend unless `write_back_grad=True`.
+  * `momentum_dtype=torch.float32` keeps an fp32 momentum buffer for bf16 parameters (the
+    reference always uses the parameter's dtype, muon_utils.py:450).
+"""
+from __future__ import annotations
+
+import logging
+from collections import OrderedDict, deque
+from itertools import chain
+from typing import Optional, Protocol
+
+import torch
+from torch import Tensor
+from torch.distributed.tensor import DTensor
+
+from . import _abi
+
+logger = logging.getLogger(__name__)
+
+NS_COEFFS = (3.4445, -4.7750, 2.0315)  # muon_utils.py:137
+
+_MUON_KEYS = {"params", "lr", "momentum", "weight_decay", "use_muon", "rms_scale", "nesterov", "ns_steps"}
+_ADAM_KEYS = {"params", "lr", "betas", "eps", "weight_decay", "use_muon"}
+
+
+# --------------------------------------------------------------------------------------
+# device plumbing
+# --------------------------------------------------------------------------------------
+def _require_cuda(t: Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise _abi.MuonHipError(f"{name} must live on a GPU: this build has no CPU path (got device {t.device})")
+
+
+def _workspace(nbytes: int, device) -> Tensor:
+    # 256-byte alignment comes with torch's caching allocator (512-byte granularity)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
+def _pointer_table(tensors, device) -> Tensor:
+    host = torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64, pin_memory=True)
+    return host.to(device, non_blocking=True)
+
+
+def scale_factor(rows: int, cols: int, rms_scale: bool) -> float:
+    """The python double apply_scaling multiplies by (muon_utils.py:167-175)."""
+    if rms_scale:
+        return 0.2 * (max(cols, rows)) ** 0.5
+    return max(1, rows / cols) ** 0.5
+
+
+# --------------------------------------------------------------------------------------
+# functional surface (muon_utils.py:95-192)
+# --------------------------------------------------------------------------------------
+def matmul_transpose_assign(d_in: Tensor, d_out: Tensor) -> None:
+    """d_out = d_in @ d_in.T on the symmetric MFMA kernel (muon_utils.py:95-119)."""
+    assert d_in.is_cuda, "Input `d_in` must be a CUDA tensor"
+    assert d_out.is_cuda, "Input `d_out` must be a CUDA tensor"
+    assert d_in.device == d_out.device, "Inputs `d_in` and `d_out` must be on the same CUDA device"
+    assert d_in.dtype == d_out.dtype, "Inputs must have the same data type"
+    assert d_in.ndim == 2, "Input `d_in` must be a 2D tensor"
+    assert d_out.ndim == 2, "Input `d_out` must be a 2D tensor"
+    assert (
+        d_in.size(0) == d_out.size(0) == d_out.size(1)
+    ), "First dimension of `d_in` must match first and second dimension of `d_out`"
+    if d_in.dtype != torch.bfloat16:
+        raise TypeError(f"the MI355X kernel multiplies bfloat16 operands, got {d_in.dtype}")
+    M, K = d_in.shape
+    geo = _abi.geometry(M, max(K, M))  # tile choice follows the small side
+    tile = geo["tile"]
+    Mp, Kp = -(-M // tile) * tile, -(-K // tile) * tile
+    with torch.cuda.device(d_in.device):
+        if (Mp, Kp) == (M, K) and d_in.is_contiguous():
+            x = d_in
+        else:
+            x = torch.zeros(Mp, Kp, dtype=torch.bfloat16, device=d_in.device)
+            x[:M, :K].copy_(d_in)
+        direct = Mp == M and d_out.is_contiguous()
+        a = d_out if direct else torch.empty(Mp, Mp, dtype=torch.bfloat16, device=d_in.device)
+        _abi.check(
+            _abi.lib().muon_hip_syrk_bf16(x.data_ptr(), a.data_ptr(), Mp, Kp, 1, _abi.CFG_AUTO,
+                                          _abi.stream_ptr(d_in.device)),
+            "syrk",
+        )
+        if not direct:
+            d_out.copy_(a[:M, :M])
+
+
+def matmul_transpose(d_in: Tensor) -> Tensor:
+    M, _ = d_in.shape
+    d_out = torch.empty((M, M), device=d_in.device, dtype=d_in.dtype)
+    matmul_transpose_assign(d_in, d_out)
+    return d_out
+
+
+def fast_newtonschulz(G: Tensor, steps: int = 5) -> Tensor:
+    """Newton-Schulz orthogonalisation (muon_utils.py:129-156); returns bf16 in G's shape.
+
+    G is 2-D, or 3-D [batch, rows, cols] for a stack of same-shape matrices (an extension:
+    one grouped dispatch per stage).
+    """
+    assert G.ndim >= 2, f"Gradient must be a 2D tensor, but got {G.shape}"
+    _require_cuda(G, "G")
+    if G.ndim > 3:
+        raise ValueError(f"expected a 2-D matrix or a 3-D stack, got shape {tuple(G.shape)}")
+    batch = G.size(0) if G.ndim == 3 else 1
+    rows, cols = G.size(-2), G.size(-1)
+    Gc = G.contiguous()
+    lib = _abi.lib()
+    a, b, c = NS_COEFFS
+    with torch.cuda.device(G.device):
+        ws = _workspace(_abi.workspace_bytes(rows, cols, batch), G.device)
+        out = torch.empty(G.shape, dtype=torch.bfloat16, device=G.device)
+        s = _abi.stream_ptr(G.device)
+        _abi.check(lib.muon_hip_cast_norm(Gc.data_ptr(), _abi.dtype_code(Gc.dtype), ws.data_ptr(), rows, cols, batch, s),
+                   "cast_norm")
+        _abi.check(lib.muon_hip_ns_grouped(ws.data_ptr(), rows, cols, batch, int(steps), a, b, c, s), "ns_grouped")
+        _abi.check(lib.muon_hip_ns_output(ws.data_ptr(), rows, cols, batch, int(steps), out.data_ptr(), s), "ns_output")
+    return out
+
+
+def apply_momentum(grad: Tensor, momentum: Tensor, beta: float, nesterov: bool) -> Tensor:
+    """In place on both tensors, as muon_utils.py:159-164; returns the update."""
+    _require_cuda(grad, "grad")
+    g2 = grad.view(len(grad), -1) if grad.ndim == 4 else grad
+    assert g2.ndim == 2 and grad.is_contiguous() and momentum.is_contiguous()
+    rows, cols = g2.shape
+    with torch.cuda.device(grad.device):
+        ws = _workspace(_abi.workspace_bytes(rows, cols, 1), grad.device)
+        gt, mt = _pointer_table([grad], grad.device), _pointer_table([momentum], grad.device)
+        _abi.check(
+            _abi.lib().muon_hip_momentum_norm(gt.data_ptr(), mt.data_ptr(), _abi.dtype_code(grad.dtype),
+                                              _abi.dtype_code(momentum.dtype), ws.data_ptr(), rows, cols, 1,
+                                              float(beta), int(bool(nesterov)), 1, _abi.stream_ptr(grad.device)),
+            "momentum_norm",
+        )
+    update = grad if nesterov else momentum
+    if update.ndim == 4:
+        update = update.view(len(update), -1)
+    return update
+
+
+def apply_scaling(grad: Tensor, rms_scale: bool = False) -> Tensor:
+    """muon_utils.py:167-175.  A host-level helper; step() fuses this into the update kernel."""
+    grad *= scale_factor(grad.size(-2), grad.size(-1), rms_scale)
+    return grad
+
+
+def muon_update(grad, momentum, beta=0.95, ns_steps=5, nesterov=True, rms_scale=False):
+    """muon_utils.py:186-192: momentum, Newton-Schulz, scaling; returns the bf16 update."""
+    update = apply_momentum(grad, momentum, beta, nesterov)
+    update = fast_newtonschulz(update, steps=ns_steps)
+    return apply_scaling(update, rms_scale)
+
+
+# --------------------------------------------------------------------------------------
+# grouped launcher
+# --------------------------------------------------------------------------------------
+def _muon_bucket_step(params, grads, moms, group, ns_steps, nesterov, write_back_grad, ws_holder, ws_limit):
+    """All stages of the Muon step for same-shape, same-dtype parameters on one device."""
+    p0 = params[0]
+    rows, cols = p0.shape
+    dev = p0.device
+    lib = _abi.lib()
+    pd, gd, md = _abi.dtype_code(p0.dtype), _abi.dtype_code(grads[0].dtype), _abi.dtype_code(moms[0].dtype)
+    a, b, c = NS_COEFFS
+    scale = scale_factor(rows, cols, group["rms_scale"])
+    n = len(params)
+    per = _abi.workspace_bytes(rows, cols, 1)
+    chunk = max(1, min(n, ws_limit // per, 65535))
+    with torch.cuda.device(dev):
+        s = _abi.stream_ptr(dev)
+        for lo in range(0, n, chunk):
+            hi = min(n, lo + chunk)
+            nb = hi - lo
+            need = _abi.workspace_bytes(rows, cols, nb)
+            ws = ws_holder.get(dev)
+            if ws is None or ws.numel() < need:
+                ws_holder[dev] = None
+                ws = ws_holder[dev] = _workspace(need, dev)
+            table = _pointer_table(params[lo:hi] + grads[lo:hi] + moms[lo:hi], dev)
+            base = table.data_ptr()
+            _abi.check(
+                lib.muon_hip_step_grouped(
+                    base, base + 8 * nb, base + 16 * nb, pd, gd, md, ws.data_ptr(), rows, cols, nb,
+                    float(group["lr"]), float(group["weight_decay"]), float(group["momentum"]), int(bool(nesterov)),
+                    int(ns_steps), float(scale), a, b, c, int(bool(write_back_grad)), s,
+                ),
+                "step_grouped",
+            )
+
+
+# --------------------------------------------------------------------------------------
+# Work protocol (muon_utils.py:195-328)
+# --------------------------------------------------------------------------------------
+class Work(Protocol):
+    def __init__(self, param, state, group, index: int):
+        ...
+
+    def start(self):
+        ...
+
+    def finish(self):
+        ...
+
+
+class _MeshWorkUnavailable:
+    """Distributed variants need collectives; this build runs on one GPU only."""
+
+    def __init__(self, param, state, group, index: int):
+        raise NotImplementedError("not implemented")
+
+
+class Fsdp1dWork(_MeshWorkUnavailable):
+    """Muon work for an FSDP2 1-D mesh (muon_utils.py:206-275): gather to an owner rank,
+    orthogonalise there, scatter back.  Not built here; the owner-side computation is
+    fast_newtonschulz on the gathered matrix."""
+
+
+class TpFsdp2dWork(_MeshWorkUnavailable):
+    """Muon work for TP + FSDP mesh (a stub in the reference too, muon_utils.py:278-284)."""
+
+
+class EpFsdp2dWork(_MeshWorkUnavailable):
+    """Muon work for EP mesh (stub, muon_utils.py:287-293)."""
+
+
+class TpEpFsdp3dWork(_MeshWorkUnavailable):
+    """Muon work for TP + EP mesh (stub, muon_utils.py:296-302)."""
+
+
+class SingelDeviceWork:
+    """Muon step for one parameter on one device (muon_utils.py:305-328): a bucket of one."""
+
+    def __init__(self, param, state, group, index: int):
+        self.param = param
+        self.state = state
+        self.group = group
+        self.reference_bug_compat = False
+        self.write_back_grad = False
+
+    def start(self):
+        g = self.group
+        ns_steps, nesterov = g["ns_steps"], g["nesterov"]
+        if self.reference_bug_compat:
+            ns_steps, nesterov = int(bool(g["nesterov"])), bool(g["ns_steps"])
+        _muon_bucket_step([self.param], [self.param.grad], [self.state["momentum_buffer"]], g, ns_steps, nesterov,
+                          self.write_back_grad, {}, 1 << 62)
+
+    def finish(self):
+        pass
+
+
+# --------------------------------------------------------------------------------------
+# the optimizer (muon_utils.py:331-482)
+# --------------------------------------------------------------------------------------
+class Muon(torch.optim.Optimizer):
+    def __init__(
+        self,
+        param_groups,
+        defaults=dict(lr=0.02),
+        is_deepspeed_enabled=False,
+        *,
+        momentum_dtype: Optional[torch.dtype] = None,
+        reference_bug_compat: bool = False,
+        write_back_grad: bool = False,
+        workspace_limit_bytes: int = 24 << 30,
+    ):
+        self.is_deepspeed_enabled = is_deepspeed_enabled
+        self.momentum_dtype = momentum_dtype
+        self.reference_bug_compat = reference_bug_compat
+        self.write_back_grad = write_back_grad
+        self.workspace_limit_bytes = int(workspace_limit_bytes)
+        self._workspaces = {}
+        for group in param_groups:
+            assert "use_muon" in group
+            if group["use_muon"]:
+                # largest first; python's sort is stable, ties keep their order
+                group["params"] = sorted(group["params"], key=lambda x: x.size(), reverse=True)
+                group["lr"] = group.get("lr", 0.02)
+                group["momentum"] = group.get("momentum", 0.95)
+                group["weight_decay"] = group.get("weight_decay", 0)
+                rms_scale = group.get("rms_scale", True)
+                if self.is_deepspeed_enabled and rms_scale:
+                    logger.warning("rms_scale for Muon is not supported in deepspeed, setting rms_scale to False")
+                    rms_scale = False
+                group["rms_scale"] = rms_scale
+                nesterov = group.get("nesterov", True)
+                if self.is_deepspeed_enabled and not nesterov:
+                    # the reference warns that it will force True and then stores False; kept as is
+                    logger.warning("disabled nesterov for Muon is not supported in deepspeed, setting nesterov to True")
+                    nesterov = False
+                group["nesterov"] = nesterov
+                group["ns_steps"] = group.get("ns_steps", 5)
+                assert set(group.keys()) == _MUON_KEYS
+            else:
+                group["lr"] = group.get("lr", 3e-4)
+                group["betas"] = group.get("betas", (0.9, 0.95))
+                group["eps"] = group.get("eps", 1e-10)
+                group["weight_decay"] = group.get("weight_decay", 0)
+                assert set(group.keys()) == _ADAM_KEYS
+        super().__init__(param_groups, defaults=defaults)
+
+    def _get_work_class(self, p: torch.Tensor) -> tuple[type[Work], int]:
+        """Work class and prefetch depth by mesh dimension (muon_utils.py:374-386)."""
+        if isinstance(p, DTensor):
+            if p.device_mesh.ndim == 1:
+                return Fsdp1dWork, 8
+            elif p.device_mesh.ndim == 2:
+                return TpFsdp2dWork, 8
+            else:
+                raise ValueError(f"Unsupported mesh dimension: {p.device_mesh.ndim}")
+        else:
+            return SingelDeviceWork, 1
+
+    @torch.no_grad()
+    def step(self, closure=None):
+        if self.is_deepspeed_enabled:
+            return self.step_deepspeed(closure)
+        else:
+            return self.step_fsdp(closure)
+
+    @torch.no_grad()
+    def step_deepspeed(self, closure=None):
+        raise NotImplementedError(
+            "the DeepSpeed branch (muon_utils.py:395-432) relies on DeepSpeed's own ZeRO Muon and is not part of "
+            "this single-GPU build"
+        )
+
+    def load_state_dict(self, state_dict) -> None:
+        """torch casts every floating state tensor to the parameter's dtype on load; put an
+        fp32 momentum buffer back when `momentum_dtype` asks for one."""
+        super().load_state_dict(state_dict)
+        if self.momentum_dtype is None:
+            return
+        saved_ids = chain.from_iterable(g["params"] for g in state_dict["param_groups"])
+        params = chain.from_iterable(g["params"] for g in self.param_groups)
+        for sid, p in zip(saved_ids, params):
+            st = state_dict["state"].get(sid)
+            if st is not None and "momentum_buffer" in st:
+                self.state[p]["momentum_buffer"] = st["momentum_buffer"].to(device=p.device, dtype=self.momentum_dtype)
+
+    def _init_muon_state(self, p: Tensor) -> dict:
+        state = self.state[p]
+        if len(state) == 0:
+            state["momentum_buffer"] = torch.zeros_like(p, dtype=self.momentum_dtype or p.dtype)
+        return state
+
+    @torch.no_grad()
+    def step_fsdp(self, closure=None):
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        dq: deque[Work] = deque()
+        for group in self.param_groups:
+            if group["use_muon"]:
+                buckets: "OrderedDict[tuple, list]" = OrderedDict()
+                for i, p in enumerate(group["params"]):
+                    assert p.ndim == 2, p.shape
+                    if p.grad is None:
+                        p.grad = torch.zeros_like(p)
+                    state = self._init_muon_state(p)
+                    class_work, prefetch_factor = self._get_work_class(p)
+                    if class_work is not SingelDeviceWork:
+                        work = class_work(p, state, group, i)
+                        work.start()
+                        dq.append(work)
+                        if len(dq) > prefetch_factor:
+                            dq.popleft().finish()
+                        continue
+                    _require_cuda(p, "a Muon parameter")
+                    if not p.is_contiguous():
+                        raise NotImplementedError("Muon parameters must be contiguous")
+                    g = p.grad if p.grad.is_contiguous() else p.grad.contiguous()
+                    m = state["momentum_buffer"]
+                    key = (p.device, tuple(p.shape), p.dtype, g.dtype, m.dtype)
+                    buckets.setdefault(key, []).append((p, g, m))
+                ns_steps, nesterov = group["ns_steps"], group["nesterov"]
+                if self.reference_bug_compat:
+                    ns_steps, nesterov = int(bool(group["nesterov"])), bool(group["ns_steps"])
+                for items in buckets.values():
+                    ps, gs, ms = (list(t) for t in zip(*items))
+                    _muon_bucket_step(ps, gs, ms, group, ns_steps, nesterov, self.write_back_grad, self._workspaces,
+                                      self.workspace_limit_bytes)
+            else:
+                for p in group["params"]:
+                    if p.grad is None:
+                        p.grad = torch.zeros_like(p)
+                    state = self.state[p]
+                    if len(state) == 0:
+                        state["exp_avg"] = torch.zeros_like(p)
+                        state["exp_avg_sq"] = torch.zeros_like(p)
+                        state["step"] = 0
+                    state["step"] += 1
+                    _adamw_tensor(p, p.grad, state["exp_avg"], state["exp_avg_sq"], state["step"], group)
+
+        for work in dq:
+            work.finish()
+
+        return loss
+
+
+def _adamw_tensor(p: Tensor, grad: Tensor, exp_avg: Tensor, exp_avg_sq: Tensor, step: int, group: dict) -> None:
+    """adam_update + decoupled decay + update (muon_utils.py:178-183, :468-477) in one kernel."""
+    _require_cuda(p, "an AdamW parameter")
+    if not (p.is_contiguous() and exp_avg.is_contiguous() and exp_avg_sq.is_contiguous()):
+        raise NotImplementedError("AdamW-fallback parameters and state must be contiguous")
+    g = grad
+    if g.dtype != p.dtype or not g.is_contiguous():
+        g = g.to(p.dtype).contiguous()
+    with torch.cuda.device(p.device):
+        _abi.check(
+            _abi.lib().muon_hip_adamw(
+                p.data_ptr(), g.data_ptr(), exp_avg.data_ptr(), exp_avg_sq.data_ptr(), _abi.dtype_code(p.dtype),
+                p.numel(), int(step), float(group["lr"]), float(group["betas"][0]), float(group["betas"][1]),
+                float(group["eps"]), float(group["weight_decay"]), _abi.stream_ptr(p.device),
+            ),
+            "adamw",
+        )
