@@ -5,6 +5,7 @@ error of the oracle computed in the same bf16 iteration order; fp32 momentum wit
 relative.  Single GEMMs are held to one bf16 ulp of the fp64 product, and to bitwise
 symmetry.
 """
+import copy
 import ctypes
 
 import pytest
@@ -38,6 +39,14 @@ def _ulp_diff_bf16(a: torch.Tensor, b: torch.Tensor) -> int:
     return (key(a.cpu()) - key(b.cpu())).abs().max().item()
 
 
+def _assert_product_close(got, ref64, absprod):
+    """One bf16 rounding of an fp32-accumulated product: within a bf16 ulp of the exact value
+    plus the accumulation error bound (which dominates where the sum cancels)."""
+    tol = ref64.abs() * 2.0 ** -8 + absprod * 2.0 ** -20
+    bad = (got.double().cpu() - ref64).abs() > tol
+    assert not bad.any(), f"{int(bad.sum())} elements outside one bf16 ulp"
+
+
 CFGS = [0, 1, 2]
 
 
@@ -54,7 +63,7 @@ def test_syrk_matches_fp64_and_is_symmetric(env, cfg, M, K, batch):
     A = A.cpu()
     assert torch.equal(A, A.mT), "X·Xᵀ must be symmetric bit for bit"
     ref64 = (X.double() @ X.double().mT)
-    assert _ulp_diff_bf16(A, ref64.bfloat16()) <= 1
+    _assert_product_close(A, ref64, X.double().abs() @ X.double().abs().mT)
     assert rel_fro(A, ref64) < 3e-3
 
 
@@ -346,7 +355,7 @@ def test_state_dict_layout_and_resume(env):
     ps[1].grad = None  # a missing grad becomes zeros
     opt.step()
     assert ps[1].grad is not None and torch.count_nonzero(ps[1].grad).item() == 0
-    sd = opt.state_dict()
+    sd = copy.deepcopy(opt.state_dict())  # state_dict() hands out the live tensors
     assert set(sd.keys()) == {"state", "param_groups"}
     assert sd["param_groups"][0]["params"] == [0, 1, 2, 3] and sd["param_groups"][1]["params"] == [4]
     assert set(sd["param_groups"][0].keys()) == {"params", "lr", "momentum", "weight_decay", "use_muon", "rms_scale", "nesterov", "ns_steps"}
@@ -411,9 +420,9 @@ def test_matmul_transpose_api(env):
     mu = env["mu"]
     X = torch.randn(200, 328, generator=torch.Generator().manual_seed(12)).bfloat16()
     out = mu.matmul_transpose(X.to(env["dev"])).cpu()
-    ref = (X.double() @ X.double().mT).bfloat16()
+    ref = X.double() @ X.double().mT
     assert out.shape == (200, 200) and torch.equal(out, out.mT)
-    assert _ulp_diff_bf16(out, ref) <= 1
+    _assert_product_close(out, ref, X.double().abs() @ X.double().abs().mT)
     with pytest.raises(AssertionError):
         mu.matmul_transpose_assign(X, torch.empty(200, 200, dtype=torch.bfloat16))  # CPU tensors
 
