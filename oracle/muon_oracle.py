@@ -141,9 +141,18 @@ def apply_scaling(update: Tensor, rms_scale: bool) -> Tensor:
 
 
 def param_update(param: Tensor, update: Tensor, lr: float, weight_decay: float) -> None:
-    """SingelDeviceWork.start's tail (muon_utils.py:324-325), in place."""
+    """SingelDeviceWork.start's tail (muon_utils.py:324-325), in place.
+
+    For a bf16 parameter the add is spelled out: ATen's GPU add kernel keeps `alpha` in fp32
+    opmath, while its CPU kernel narrows alpha to bf16 first (measured: -0.02 becomes
+    -0.02002).  The reference runs on a GPU, so the GPU arithmetic is the one restated.
+    """
     param.mul_(1 - lr * weight_decay)
-    param.add_(update.reshape(param.shape), alpha=-lr)
+    update = update.reshape(param.shape)
+    if param.dtype == torch.float32:
+        param.add_(update, alpha=-lr)
+    else:
+        param.copy_((param.float() + _f32(-lr) * update.float()).to(param.dtype))
 
 
 def muon_step_matrix(
@@ -196,8 +205,7 @@ def adam_update(grad: Tensor, buf1: Tensor, buf2: Tensor, step: int, betas, eps:
 def adamw_step_tensor(param, grad, exp_avg, exp_avg_sq, step, lr, betas, eps, weight_decay) -> None:
     """Adam branch of step_fsdp (muon_utils.py:468-477), in place. `step` is already incremented."""
     upd = adam_update(grad, exp_avg, exp_avg_sq, step, betas, eps)
-    param.mul_(1 - lr * weight_decay)
-    param.add_(upd, alpha=-lr)
+    param_update(param, upd, lr, weight_decay)
 
 
 class OracleMuon:

@@ -455,3 +455,39 @@ def test_config2_full_size_sampled_parity(env):
         # so ||o||_F^2 is close to min(rows, cols) (times the shape scale squared)
     for i, p in enumerate(gp):
         assert torch.isfinite(p).all()
+
+
+def test_golden_vectors_on_gpu(env):
+    """The committed golden vectors (tests/golden/, written by make_fixtures.py from the oracle)."""
+    import os
+
+    import numpy as np
+
+    from tests.golden.make_fixtures import STEP_SPEC
+    from tests.helpers import bf16_from_u16
+
+    mu = env["mu"]
+    gdir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    data = np.load(os.path.join(gdir, "ns_small.npz"))
+    for key in data.files:
+        _, shape, seed, steps = key.split("_")
+        rows, cols = (int(v) for v in shape.split("x"))
+        G = torch.randn(rows, cols, generator=torch.Generator().manual_seed(int(seed[4:])))
+        got = mu.fast_newtonschulz(G.to(env["dev"]), int(steps[5:]))
+        assert rel_fro(got, bf16_from_u16(data[key])) <= (NS_TOL if steps == "steps5" else 2e-3), key
+    data = np.load(os.path.join(gdir, "step_small.npz"))
+    weights, grads = make_param_set(STEP_SPEC, layers=1, seed=7, steps=3)
+    params = [torch.nn.Parameter(w.clone().to(env["dev"])) for _, w in weights]
+    opt = mu.Muon([dict(params=list(params), use_muon=True, **MUON_HP)])
+    lr, wd = MUON_HP["lr"], MUON_HP["weight_decay"]
+    for step in range(3):
+        for p, g in zip(params, grads[step]):
+            p.grad = g.to(env["dev"])
+        before = [p.detach().clone() for p in opt.param_groups[0]["params"]]
+        opt.step()
+        for j, p in enumerate(opt.param_groups[0]["params"]):
+            o_gpu = (before[j].double().cpu() * (1 - lr * wd) - p.detach().double().cpu()) / lr
+            assert rel_fro(o_gpu, bf16_from_u16(data[f"step{step}_update{j}"])) <= NS_TOL
+    for j, p in enumerate(opt.param_groups[0]["params"]):
+        assert rel_fro(opt.state[p]["momentum_buffer"], torch.from_numpy(data[f"final_momentum{j}"])) <= MOM_TOL
+        assert rel_fro(p.detach(), torch.from_numpy(data[f"final_param{j}"])) <= 2e-3

@@ -1,0 +1,166 @@
+"""Host-side contract of the Muon drop-in, checked without a GPU: constructor defaults,
+asserts and sort order (muon_utils.py:332-372), work-class dispatch (:374-386), the loud
+failure when tensors are not on a GPU, and that libmuon_hip.so loads and exports every
+symbol include/muon_hip.h declares (no compute calls here)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from lmms_engine_amd import _abi, muon_utils
+from lmms_engine_amd.muon_utils import Muon
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def P(*shape):
+    return torch.nn.Parameter(torch.zeros(*shape))
+
+
+def test_muon_group_defaults_and_keys():
+    g = dict(params=[P(4, 3)], use_muon=True)
+    opt = Muon([g])
+    assert g["lr"] == 0.02 and g["momentum"] == 0.95 and g["weight_decay"] == 0
+    assert g["rms_scale"] is True and g["nesterov"] is True and g["ns_steps"] == 5
+    assert set(g.keys()) == {"params", "lr", "momentum", "weight_decay", "use_muon", "rms_scale", "nesterov", "ns_steps"}
+    assert opt.defaults == dict(lr=0.02) and opt.is_deepspeed_enabled is False
+    assert opt.param_groups[0] is g or opt.param_groups[0]["params"][0] is g["params"][0]
+
+
+def test_adam_group_defaults_and_keys():
+    g = dict(params=[P(7)], use_muon=False)
+    Muon([g])
+    assert g["lr"] == 3e-4 and g["betas"] == (0.9, 0.95) and g["eps"] == 1e-10 and g["weight_decay"] == 0
+    assert set(g.keys()) == {"params", "lr", "betas", "eps", "weight_decay", "use_muon"}
+
+
+def test_given_values_are_kept():
+    g = dict(params=[P(4, 3)], use_muon=True, lr=1e-3, momentum=0.9, weight_decay=0.1, rms_scale=False, nesterov=False,
+             ns_steps=3)
+    Muon([g], defaults=dict(lr=1e-3))
+    assert (g["lr"], g["momentum"], g["weight_decay"], g["rms_scale"], g["nesterov"], g["ns_steps"]) == (1e-3, 0.9, 0.1, False, False, 3)
+
+
+def test_asserts():
+    with pytest.raises(AssertionError):
+        Muon([dict(params=[P(4, 3)])])  # use_muon missing
+    with pytest.raises(AssertionError):
+        Muon([dict(params=[P(4, 3)], use_muon=True, betas=(0.9, 0.95))])  # foreign key in a Muon group
+    with pytest.raises(AssertionError):
+        Muon([dict(params=[P(4)], use_muon=False, momentum=0.9)])  # foreign key in an Adam group
+
+
+def test_params_sorted_by_size_descending_and_stable():
+    ps = [P(2, 3), P(5, 1), P(2, 3), P(5, 4)]
+    opt = Muon([dict(params=list(ps), use_muon=True)])
+    got = opt.param_groups[0]["params"]
+    assert [tuple(p.shape) for p in got] == [(5, 4), (5, 1), (2, 3), (2, 3)]
+    assert got[2] is ps[0] and got[3] is ps[2], "ties keep their order"
+
+
+def test_trainer_factory_shaped_groups_with_empty_lists():
+    """The four dicts Trainer.create_optimizer builds (train/hf/trainer.py:417-448), some empty."""
+    w, e = P(8, 8), P(10)
+    groups = [
+        dict(params=[], use_muon=True, lr=1e-3, momentum=0.95, weight_decay=0.01),
+        dict(params=[w], use_muon=True, lr=1e-3, momentum=0.95, weight_decay=0.0),
+        dict(params=[], use_muon=False, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01),
+        dict(params=[e], use_muon=False, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0),
+    ]
+    opt = Muon(groups, defaults=dict(lr=1e-3), is_deepspeed_enabled=False)
+    assert len(opt.param_groups) == 4
+    sd = opt.state_dict()
+    assert sd["state"] == {} and [g["params"] for g in sd["param_groups"]] == [[], [0], [], [1]]
+
+
+def test_deepspeed_quirks_kept():
+    g = dict(params=[P(4, 3)], use_muon=True, nesterov=False)
+    opt = Muon([g], is_deepspeed_enabled=True)
+    assert g["rms_scale"] is False, "DeepSpeed forces rms_scale off"
+    assert g["nesterov"] is False, "the reference warns but keeps False"
+    with pytest.raises(NotImplementedError):
+        opt.step()
+
+
+def test_work_class_dispatch():
+    opt = Muon([dict(params=[P(4, 3)], use_muon=True)])
+    cls, prefetch = opt._get_work_class(torch.zeros(2, 2))
+    assert cls is muon_utils.SingelDeviceWork and prefetch == 1
+    for stub in (muon_utils.Fsdp1dWork, muon_utils.TpFsdp2dWork, muon_utils.EpFsdp2dWork, muon_utils.TpEpFsdp3dWork):
+        with pytest.raises(NotImplementedError):
+            stub(None, None, None, 0)
+
+
+def test_cpu_tensors_fail_loudly():
+    p = P(4, 3)
+    p.grad = torch.zeros(4, 3)
+    opt = Muon([dict(params=[p], use_muon=True)])
+    with pytest.raises(_abi.MuonHipError, match="no CPU path"):
+        opt.step()
+    q = P(5)
+    q.grad = torch.zeros(5)
+    with pytest.raises(_abi.MuonHipError, match="no CPU path"):
+        Muon([dict(params=[q], use_muon=False)]).step()
+    with pytest.raises(_abi.MuonHipError):
+        muon_utils.fast_newtonschulz(torch.zeros(4, 4))
+    with pytest.raises(AssertionError):
+        muon_utils.matmul_transpose(torch.zeros(4, 4, dtype=torch.bfloat16))
+
+
+def test_non_2d_muon_param_asserts_before_any_kernel():
+    p = P(5)
+    p.grad = torch.zeros(5)
+    with pytest.raises(AssertionError):
+        Muon([dict(params=[p], use_muon=True)]).step()
+
+
+def test_scale_factor():
+    assert muon_utils.scale_factor(4864, 896, False) == (4864 / 896) ** 0.5
+    assert muon_utils.scale_factor(896, 4864, False) == 1.0
+    assert muon_utils.scale_factor(896, 4864, True) == 0.2 * 4864 ** 0.5
+
+
+def test_missing_library_is_an_error(monkeypatch):
+    monkeypatch.setattr(_abi, "_lib", None)
+    monkeypatch.setattr(_abi, "LIB_PATH", "/nonexistent/libmuon_hip.so")
+    with pytest.raises(_abi.MuonHipError, match="no fallback"):
+        _abi.lib()
+
+
+# ---- the C ABI ----------------------------------------------------------------------------
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "muon_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(muon_hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = _declared_symbols()
+    assert len(names) >= 17
+    lib = ctypes.CDLL(_abi.LIB_PATH)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/muon_hip.h but not exported"
+    assert set(names) == set(_abi.SIGNATURES), "the ctypes table mirrors the header one to one"
+
+
+def test_host_only_entry_points():
+    lib = _abi.lib()
+    assert lib.muon_hip_version() >= 100
+    geo = _abi.geometry(896, 4864)
+    assert geo == dict(M=896, K=4864, Mp=896, Kp=4864, tile=128)
+    geo = _abi.geometry(12288, 4096)
+    assert (geo["M"], geo["K"], geo["tile"]) == (4096, 12288, 256)
+    assert _abi.geometry(100, 300) == dict(M=100, K=300, Mp=128, Kp=384, tile=128)
+    w1, w2 = _abi.workspace_bytes(896, 4864, 1), _abi.workspace_bytes(896, 4864, 2)
+    assert w1 >= 8 * 896 * 4864 + 4 * 896 * 896 and w1 < w2 <= 2 * w1
+    assert lib.muon_hip_workspace_bytes(0, 4, 1) == 0 and b"positive" in lib.muon_hip_last_error()
+    assert lib.muon_hip_set_gemm_config(7) == -1
+    assert lib.muon_hip_set_gemm_config(_abi.CFG_256x256_W4) == 0
+    try:
+        assert _abi.geometry(896, 4864)["tile"] == 256 and _abi.geometry(896, 4864)["Mp"] == 1024
+    finally:
+        assert lib.muon_hip_set_gemm_config(_abi.CFG_AUTO) == 0
+    with pytest.raises(TypeError):
+        _abi.dtype_code(torch.float16)
