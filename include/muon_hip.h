@@ -52,6 +52,10 @@ extern "C" {
 #define MUON_HIP_CFG_128x128_W4 0
 #define MUON_HIP_CFG_256x256_W4 1
 #define MUON_HIP_CFG_256x256_W8 2
+/* the same tiles fed by direct global->LDS loads (global_load_lds_dwordx4) */
+#define MUON_HIP_CFG_128x128_W4_DLDS 3
+#define MUON_HIP_CFG_256x256_W4_DLDS 4
+#define MUON_HIP_CFG_256x256_W8_DLDS 5
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);

@@ -16,6 +16,8 @@ LIB_PATH = os.path.join(_HERE, "libmuon_hip.so")
 
 F32, BF16 = 0, 1
 CFG_AUTO, CFG_128x128_W4, CFG_256x256_W4, CFG_256x256_W8 = -1, 0, 1, 2
+CFG_128x128_W4_DLDS, CFG_256x256_W4_DLDS, CFG_256x256_W8_DLDS = 3, 4, 5
+GEMM_CONFIGS = [0, 1, 2, 3, 4, 5]
 K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW = range(7)
 KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw"]
 

@@ -4,7 +4,15 @@
 #include "common.h"
 
 enum { EPI_SYRK = 0, EPI_SYMPOLY = 1, EPI_BX = 2 };
-enum { GEMM_CFG_128x128_W4 = 0, GEMM_CFG_256x256_W4 = 1, GEMM_CFG_256x256_W8 = 2, GEMM_CFG_COUNT = 3 };
+enum {
+    GEMM_CFG_128x128_W4 = 0,
+    GEMM_CFG_256x256_W4 = 1,
+    GEMM_CFG_256x256_W8 = 2,
+    GEMM_CFG_128x128_W4_DLDS = 3,
+    GEMM_CFG_256x256_W4_DLDS = 4,
+    GEMM_CFG_256x256_W8_DLDS = 5,
+    GEMM_CFG_COUNT = 6
+};
 
 struct GemmArgs {
     const bf16_t* P;   // left operand rows (reduction contiguous)

@@ -60,6 +60,77 @@ __device__ __forceinline__ void rect_decode(int t, int TM, int TN, int& ti, int&
     tj = r / gm;
 }
 
+struct TileCoord {
+    int bidx, ti, tj;
+};
+
+template <int EPI>
+__device__ __forceinline__ TileCoord decode_tile(const GemmArgs& g) {
+    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+    TileCoord tc;
+    tc.bidx = logical / g.tiles_per_mat;
+    const int t = logical - tc.bidx * g.tiles_per_mat;
+    if (EPI == EPI_BX) rect_decode<4>(t, g.tiles_m, g.tiles_n, tc.ti, tc.tj);
+    else tri_decode<4>(t, g.tiles_m, tc.ti, tc.tj);
+    return tc;
+}
+
+// Lane (lane&31) owns column j; registers 4q..4q+3 are rows 8q + 4*(lane>>5) + 0..3.
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
+                                         f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32]) {
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WGN, wn = wave % WGN, hi = lane >> 5;
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+    const bool diag = (EPI != EPI_BX) && (tc.ti == tc.tj);
+    bf16_t* C = g.C ? g.C + tc.bidx * g.strideC : nullptr;
+    bf16_t* Ct = g.Ct ? g.Ct + tc.bidx * g.strideCt : nullptr;
+    const bf16_t* Et = g.Et ? g.Et + tc.bidx * g.strideEt : nullptr;
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const long gj = n0 + wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const long gi = m0 + wm * WTM + i * 32 + q * 8 + hi * 4;
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = rbf(acc[i][j][q * 4 + r]);
+                if (EPI != EPI_SYRK) {
+                    const bf16x4 e = *(const bf16x4*)(Et + gj * g.ldet + gi);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (EPI == EPI_SYMPOLY) v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + rbf(g.s1 * v[r]));
+                        else v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + v[r]);
+                    }
+                }
+                bf16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = f2bf(v[r]);
+                if (diag) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (gi + r <= gj) {
+                            C[(gi + r) * g.ldc + gj] = o[r];
+                            C[gj * g.ldc + gi + r] = o[r];
+                        }
+                    }
+                } else {
+                    if (C) {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) C[(gi + r) * g.ldc + gj] = o[r];
+                    }
+                    if (Ct) *(bf16x4*)(Ct + gj * g.ldct + gi) = o;
+                }
+            }
+        }
+    }
+}
+
+// ---- variant 1: global -> registers -> LDS, two LDS stages, one barrier per k-tile -------
 template <int BM, int BN, int WGM, int WGN, int EPI>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g) {
     constexpr int NT = WGM * WGN * 64;
@@ -76,19 +147,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
+    const TileCoord tc = decode_tile<EPI>(g);
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+    const bf16_t* Pb = g.P + tc.bidx * g.strideP + m0 * g.ldp;
+    const bf16_t* Qb = g.Q + tc.bidx * g.strideQ + n0 * g.ldq;
 
-    const int logical = xcd_remap(blockIdx.x, gridDim.x);
-    const int bidx = logical / g.tiles_per_mat;
-    const int t = logical - bidx * g.tiles_per_mat;
-    int ti, tj;
-    if (EPI == EPI_BX) rect_decode<4>(t, g.tiles_m, g.tiles_n, ti, tj);
-    else tri_decode<4>(t, g.tiles_m, ti, tj);
-
-    const long m0 = (long)ti * BM, n0 = (long)tj * BN;
-    const bf16_t* Pb = g.P + bidx * g.strideP + m0 * g.ldp;
-    const bf16_t* Qb = g.Q + bidx * g.strideQ + n0 * g.ldq;
-
-    // ---- global -> register -> LDS staging -------------------------------------------
     const int lrow = tid >> 3, lc = tid & 7;
     const bf16_t* pa = Pb + (long)lrow * g.ldp + lc * 8;
     const bf16_t* pb = Qb + (long)lrow * g.ldq + lc * 8;
@@ -148,60 +211,165 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g
         if (more) lstore((kt + 1) & 1);
         __syncthreads();
     }
-
-    // ---- epilogue ---------------------------------------------------------------------
-    // Lane (lane&31) owns column j; registers 4q..4q+3 are rows 8q + 4*(lane>>5) + 0..3.
-    const bool diag = (EPI != EPI_BX) && (ti == tj);
-    bf16_t* C = g.C ? g.C + bidx * g.strideC : nullptr;
-    bf16_t* Ct = g.Ct ? g.Ct + bidx * g.strideCt : nullptr;
-    const bf16_t* Et = g.Et ? g.Et + bidx * g.strideEt : nullptr;
-#pragma unroll
-    for (int i = 0; i < FM; ++i) {
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-            const long gj = n0 + wn * WTN + j * 32 + (lane & 31);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const long gi = m0 + wm * WTM + i * 32 + q * 8 + hi * 4;
-                float v[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) v[r] = rbf(acc[i][j][q * 4 + r]);
-                if (EPI != EPI_SYRK) {
-                    const bf16x4 e = *(const bf16x4*)(Et + gj * g.ldet + gi);
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        if (EPI == EPI_SYMPOLY) v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + rbf(g.s1 * v[r]));
-                        else v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + v[r]);
-                    }
-                }
-                bf16x4 o;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) o[r] = f2bf(v[r]);
-                if (diag) {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        if (gi + r <= gj) {
-                            C[(gi + r) * g.ldc + gj] = o[r];
-                            C[gj * g.ldc + gi + r] = o[r];
-                        }
-                    }
-                } else {
-                    if (C) {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) C[(gi + r) * g.ldc + gj] = o[r];
-                    }
-                    if (Ct) *(bf16x4*)(Ct + gj * g.ldct + gi) = o;
-                }
-            }
-        }
-    }
+#ifdef EXP_NO_EPI
+    float ssum = 0.f;
+    for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
+    if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
+#else
+    epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc);
+#endif
 }
 
+// ---- variant 2: global -> LDS directly (global_load_lds_dwordx4), two LDS stages ---------
+// One wave-level load instruction fills 1 KB of LDS in lane order, i.e. 8 rows of the tile;
+// the XOR swizzle is applied on the global side: lane L fetches the chunk whose swizzled
+// position is L&7.  Loads for k-tile t+2 are issued as soon as every wave has finished
+// reading k-tile t, and are waited for (vmcnt) one whole tile of MFMA work later.
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+typedef const __attribute__((address_space(1))) void* glb_void_ptr;
+
+#define WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
+// s_waitcnt with only vmcnt set: vmcnt is split over bits [3:0] and [15:14] (N < 64)
+#define WAIT_VM(N) __builtin_amdgcn_s_waitcnt(0x0F70 | ((N) & 15) | (((N) >> 4) << 14))
+
 template <int BM, int BN, int WGM, int WGN, int EPI>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_dlds_kernel(const GemmArgs g) {
+    constexpr int NW = WGM * WGN;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE = A_BYTES + B_BYTES;
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;  // 1 KB load instructions per wave per k-tile
+    constexpr int KS = BK / 16;
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "dma split");
+    static_assert(LA + LB < 64, "vmcnt immediate");
+    static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const TileCoord tc = decode_tile<EPI>(g);
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+    const bf16_t* Pb = g.P + tc.bidx * g.strideP + m0 * g.ldp;
+    const bf16_t* Qb = g.Q + tc.bidx * g.strideQ + n0 * g.ldq;
+
+    // Wave w fills rows [w*8*LA, +8*LA) of A and [w*8*LB, +8*LB) of B, 8 rows per instruction.
+    // Row r keeps chunk c at position c ^ ((r>>1)&7); lane L lands on position L&7 of row
+    // r = 8*group + (L>>3), so it fetches chunk (L&7) ^ (4*(group&1) + (L>>4)).
+    const int drow = lane >> 3;
+    const bf16_t* pa = Pb + (long)(wave * 8 * LA + drow) * g.ldp;
+    const bf16_t* pb = Qb + (long)(wave * 8 * LB + drow) * g.ldq;
+    const int lds_a = wave * 8 * LA * ROW_BYTES;
+    const int lds_b = A_BYTES + wave * 8 * LB * ROW_BYTES;
+    const int ch_even = ((lane & 7) ^ (drow >> 1)) * 8, ch_odd = ((lane & 7) ^ (4 | (drow >> 1))) * 8;
+
+    auto issue = [&](int stage, int k0) {
+        unsigned char* s = smem + stage * STAGE;
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            const int ch = ((wave * LA + i) & 1) ? ch_odd : ch_even;
+            __builtin_amdgcn_global_load_lds((glb_void_ptr)(pa + (long)i * 8 * g.ldp + k0 + ch),
+                                             (lds_void_ptr)(s + lds_a + i * 8 * ROW_BYTES), 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < LB; ++i) {
+            const int ch = ((wave * LB + i) & 1) ? ch_odd : ch_even;
+            __builtin_amdgcn_global_load_lds((glb_void_ptr)(pb + (long)i * 8 * g.ldq + k0 + ch),
+                                             (lds_void_ptr)(s + lds_b + i * 8 * ROW_BYTES), 16, 0, 0);
+        }
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int sw = (lane >> 1) & 7, hi = lane >> 5;
+    const int a_off = (wm * WTM + (lane & 31)) * ROW_BYTES;
+    const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROW_BYTES;
+
+    const int nk = g.kdim / BK;
+#ifdef EXP_DEPTH
+    for (int d = 0; d < EXP_DEPTH; ++d) issue(d & 1, d * BK);
+#else
+    issue(0, 0);
+    if (nk > 1) issue(1, BK);
+#endif
+    for (int kt = 0; kt < nk; ++kt) {
+        // k-tile kt has landed once at most the next tile's loads are still in flight
+#ifdef EXP_DEPTH
+        if (kt + EXP_DEPTH <= nk) WAIT_VM((EXP_DEPTH - 1) * (LA + LB));
+        else WAIT_VM(0);
+#elif !defined(EXP_NO_DMA)
+        if (kt + 1 < nk) WAIT_VM(LA + LB);
+        else WAIT_VM(0);
+#endif
+#ifndef EXP_NO_BARRIER
+        __builtin_amdgcn_s_barrier();
+#endif
+        asm volatile("" ::: "memory");
+        const unsigned char* st = smem + (kt & 1) * STAGE;
+        bf16x8 af[2][FM], bq[2][FN];
+        auto lfrag = [&](int buf, int ks) {
+            const int co = (((ks << 1) | hi) ^ sw) << 4;
+#pragma unroll
+            for (int i = 0; i < FM; ++i) af[buf][i] = *(const bf16x8*)(st + a_off + i * 32 * ROW_BYTES + co);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) bq[buf][j] = *(const bf16x8*)(st + b_off + j * 32 * ROW_BYTES + co);
+        };
+        lfrag(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            // the LDS reads of the next k-step go out before this k-step's MFMAs start, so
+            // their latency hides behind FM*FN MFMAs; the fences keep the scheduler from
+            // sinking them back next to their uses
+#ifndef EXP_NO_LDS
+            if (ks + 1 < KS) lfrag((ks + 1) & 1, ks + 1);
+#endif
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+#ifndef EXP_NO_MFMA
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[ks & 1][i], bq[ks & 1][j], acc[i][j], 0, 0, 0);
+#else
+                    acc[i][j][0] += (float)af[ks & 1][i][0] * (float)bq[ks & 1][j][0];
+#endif
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (kt + 2 < nk) {
+            // every wave must be done reading this stage before new data may land in it
+            WAIT_LGKM0();
+            asm volatile("" ::: "memory");
+#ifndef EXP_NO_BARRIER
+            __builtin_amdgcn_s_barrier();
+#endif
+#ifdef EXP_DEPTH
+            if (kt + EXP_DEPTH < nk) issue((kt + EXP_DEPTH) & 1, (kt + EXP_DEPTH) * BK);
+#elif !defined(EXP_NO_DMA)
+            issue(kt & 1, (kt + 2) * BK);
+#endif
+        }
+    }
+#ifdef EXP_NO_EPI
+    float ssum = 0.f;
+    for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
+    if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
+#else
+    epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc);
+#endif
+}
+
+template <int BM, int BN, int WGM, int WGN, int EPI, bool DLDS>
 hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
     constexpr int smem = 2 * (BM + BN) * ROW_BYTES;
     static bool configured = false;  // per instantiation; the attribute is idempotent
-    auto kern = gemm_nt_kernel<BM, BN, WGM, WGN, EPI>;
+    auto kern = DLDS ? gemm_nt_dlds_kernel<BM, BN, WGM, WGN, EPI> : gemm_nt_kernel<BM, BN, WGM, WGN, EPI>;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
@@ -214,9 +382,12 @@ hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
 template <int EPI>
 hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t stream) {
     switch (cfg) {
-        case GEMM_CFG_128x128_W4: return launch_one<128, 128, 2, 2, EPI>(g, nblocks, stream);
-        case GEMM_CFG_256x256_W4: return launch_one<256, 256, 2, 2, EPI>(g, nblocks, stream);
-        case GEMM_CFG_256x256_W8: return launch_one<256, 256, 2, 4, EPI>(g, nblocks, stream);
+        case GEMM_CFG_128x128_W4: return launch_one<128, 128, 2, 2, EPI, false>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W4: return launch_one<256, 256, 2, 2, EPI, false>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8: return launch_one<256, 256, 2, 4, EPI, false>(g, nblocks, stream);
+        case GEMM_CFG_128x128_W4_DLDS: return launch_one<128, 128, 2, 2, EPI, true>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W4_DLDS: return launch_one<256, 256, 2, 2, EPI, true>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8_DLDS: return launch_one<256, 256, 2, 4, EPI, true>(g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -225,9 +396,12 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
 
 int gemm_cfg_tile(int cfg) {
     switch (cfg) {
-        case GEMM_CFG_128x128_W4: return 128;
+        case GEMM_CFG_128x128_W4:
+        case GEMM_CFG_128x128_W4_DLDS: return 128;
         case GEMM_CFG_256x256_W4:
-        case GEMM_CFG_256x256_W8: return 256;
+        case GEMM_CFG_256x256_W8:
+        case GEMM_CFG_256x256_W4_DLDS:
+        case GEMM_CFG_256x256_W8_DLDS: return 256;
         default: return 0;
     }
 }
