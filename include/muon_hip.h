@@ -56,6 +56,13 @@ extern "C" {
 #define MUON_HIP_CFG_128x128_W4_DLDS 3
 #define MUON_HIP_CFG_256x256_W4_DLDS 4
 #define MUON_HIP_CFG_256x256_W8_DLDS 5
+/* direct loads, software pipelined: MFMAs interleaved with LDS reads and loads, one barrier per k-tile */
+#define MUON_HIP_CFG_128x128_W4_PIPE 6
+#define MUON_HIP_CFG_256x256_W4_PIPE 7
+#define MUON_HIP_CFG_256x256_W8_PIPE 8
+/* 32-column k-tiles in four LDS stages: loads spread evenly between the MFMAs */
+#define MUON_HIP_CFG_128x128_W4_PIPE4 9
+#define MUON_HIP_CFG_256x256_W4_PIPE4 10
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);
@@ -112,20 +119,26 @@ int muon_hip_step_grouped(const void* const* p_ptrs, const void* const* g_ptrs, 
                           double lr, double weight_decay, double beta, int nesterov, int ns_steps, double scale,
                           double a, double b, double c, int write_back_grad, void* stream);
 
-/* ---- single GEMM entry points (explicit buffers, already padded to whole tiles) ------- */
+/* ---- single GEMM entry points (explicit buffers, already padded to whole tiles) -------
+ * Every matrix is row-major with a row pitch `ld*` in elements (>= its width, a multiple of
+ * 8); matrix b of a batch starts at b * rows * ld.  Pitches that are multiples of 2048
+ * elements are legal but slow (all rows of a tile share an L2 channel): add 128. */
 
-/* A[batch][Mp][Mp] = bf16(X Xt) for X[batch][Mp][Kp]: matmul_transpose_assign + mmt_kernel,
- * muon_utils.py:95-119 and :28-92.  Upper tiles computed, mirrored below the diagonal. */
-int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* stream);
+/* A[batch][Mp][lda] = bf16(X Xt) for X[batch][Mp][ldx] (Kp columns used):
+ * matmul_transpose_assign + mmt_kernel, muon_utils.py:95-119 and :28-92.  Upper tiles
+ * computed, mirrored below the diagonal. */
+int muon_hip_syrk_bf16(const void* X, int ldx, void* A, int lda, int Mp, int Kp, int batch, int cfg, void* stream);
 
-/* B = bf16(bf16(b*A) + bf16(c*bf16(A A))) for symmetric A: muon_utils.py:150-151. */
-int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* stream);
+/* B = bf16(bf16(b*A) + bf16(c*bf16(A A))) for symmetric A: muon_utils.py:150-151.
+ * A and B share the pitch lda. */
+int muon_hip_sympoly_bf16(const void* A, void* B, int lda, int Mp, int batch, double b, double c, int cfg,
+                          void* stream);
 
-/* X' = bf16(bf16(a*X) + bf16(B X)): muon_utils.py:152.  B[batch][Mp][Mp] symmetric,
- * XT[batch][Kp][Mp] the transposed copy of X; writes Xout[batch][Mp][Kp] and/or
- * XTout[batch][Kp][Mp] (either may be null, not both). */
-int muon_hip_bx_axpy_bf16(const void* B, const void* XT, void* Xout, void* XTout, int Mp, int Kp, int batch,
-                          double a, int cfg, void* stream);
+/* X' = bf16(bf16(a*X) + bf16(B X)): muon_utils.py:152.  B[batch][Mp][lda] symmetric,
+ * XT[batch][Kp][ldxt] the transposed copy of X; writes Xout[batch][Mp][ldx] and/or
+ * XTout[batch][Kp][ldxt] (either may be null, not both). */
+int muon_hip_bx_axpy_bf16(const void* B, int lda, const void* XT, int ldxt, void* Xout, int ldx, void* XTout, int Mp,
+                          int Kp, int batch, double a, int cfg, void* stream);
 
 /* ---- AdamW fallback ------------------------------------------------------------------ */
 

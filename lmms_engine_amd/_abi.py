@@ -17,7 +17,9 @@ LIB_PATH = os.path.join(_HERE, "libmuon_hip.so")
 F32, BF16 = 0, 1
 CFG_AUTO, CFG_128x128_W4, CFG_256x256_W4, CFG_256x256_W8 = -1, 0, 1, 2
 CFG_128x128_W4_DLDS, CFG_256x256_W4_DLDS, CFG_256x256_W8_DLDS = 3, 4, 5
-GEMM_CONFIGS = [0, 1, 2, 3, 4, 5]
+CFG_128x128_W4_PIPE, CFG_256x256_W4_PIPE, CFG_256x256_W8_PIPE = 6, 7, 8
+CFG_128x128_W4_PIPE4, CFG_256x256_W4_PIPE4 = 9, 10
+GEMM_CONFIGS = list(range(11))
 K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW = range(7)
 KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw"]
 
@@ -38,10 +40,10 @@ SIGNATURES = {
     "muon_hip_step_grouped": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int,
                                       c_double, c_double, c_double, c_int, c_int, c_double, c_double, c_double,
                                       c_double, c_int, c_void_p]),
-    "muon_hip_syrk_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
-    "muon_hip_sympoly_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_double, c_double, c_int, c_void_p]),
-    "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_int,
-                                      c_void_p]),
+    "muon_hip_syrk_bf16": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "muon_hip_sympoly_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_double, c_int, c_void_p]),
+    "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
+                                      c_double, c_int, c_void_p]),
     "muon_hip_adamw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_double,
                                c_double, c_double, c_double, c_void_p]),
     "muon_hip_timing_enable": (c_int, [c_int]),

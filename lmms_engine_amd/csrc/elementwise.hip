@@ -153,8 +153,8 @@ __device__ __forceinline__ float frob_denominator(const float* part, int nparts,
 // One 64x64 tile of the padded operand X (Mp x Kp) and of its transposed copy Xt (Kp x Mp)
 // from the bf16 blend u held in the parameter's own layout (rows x cols).
 __global__ void __launch_bounds__(256)
-normalize_kernel(const bf16_t* U, long strideU, const float* partials, int nparts, bf16_t* X, bf16_t* XT,
-                 long strideX, int rows, int cols, int Mp, int Kp) {
+normalize_kernel(const bf16_t* U, long strideU, const float* partials, int nparts, bf16_t* X, int ldx, long strideX,
+                 bf16_t* XT, int ldxt, long strideXT, int rows, int cols, int Mp, int Kp) {
     __shared__ float red[4];
     __shared__ __align__(16) bf16_t tile[64][72];
     const int b = blockIdx.y;
@@ -163,9 +163,10 @@ normalize_kernel(const bf16_t* U, long strideU, const float* partials, int npart
     // The tile is addressed in the parameter's orientation: r over rows, c over cols.
     // transposed (rows > cols): X = u^T, so the padded row-major image of u is Xt.
     const bool transposed = rows > cols;
-    const int Rp = transposed ? Kp : Mp, Cp = transposed ? Mp : Kp;  // padded rows/cols of u's image
-    bf16_t* same = (transposed ? XT : X) + b * strideX;               // same orientation as u
-    bf16_t* flip = (transposed ? X : XT) + b * strideX;               // the transposed image
+    const int Cp = transposed ? Mp : Kp;                                  // padded cols of u's image
+    bf16_t* same = transposed ? XT + b * strideXT : X + b * strideX;      // same orientation as u
+    bf16_t* flip = transposed ? X + b * strideX : XT + b * strideXT;      // the transposed image
+    const int ld_same = transposed ? ldxt : ldx, ld_flip = transposed ? ldx : ldxt;
     const int tiles_c = Cp / 64;
     const int r0 = (blockIdx.x / tiles_c) * 64, c0 = (blockIdx.x % tiles_c) * 64;
     const int tr = threadIdx.x >> 3, tc = (threadIdx.x & 7) * 8;
@@ -187,7 +188,7 @@ normalize_kernel(const bf16_t* U, long strideU, const float* partials, int npart
             }
         }
         *(bf16x8*)(&tile[tr + h * 32][tc]) = o;
-        *(bf16x8*)(same + (long)r * Cp + c) = o;
+        *(bf16x8*)(same + (long)r * ld_same + c) = o;
     }
     __syncthreads();
 #pragma unroll
@@ -197,7 +198,7 @@ normalize_kernel(const bf16_t* U, long strideU, const float* partials, int npart
         bf16x8 o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[i] = tile[fr + i][fc];
-        *(bf16x8*)(flip + (long)(c0 + fc) * Rp + r0 + fr) = o;
+        *(bf16x8*)(flip + (long)(c0 + fc) * ld_flip + r0 + fr) = o;
     }
 }
 
@@ -334,11 +335,12 @@ hipError_t launch_cast_norm(const void* G, long strideG, int g_dtype, bf16_t* U,
     return hipGetLastError();
 }
 
-hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, bf16_t* X, bf16_t* XT,
-                            long strideX, int rows, int cols, int Mp, int Kp, int batch, hipStream_t stream) {
+hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, bf16_t* X, int ldx,
+                            long strideX, bf16_t* XT, int ldxt, long strideXT, int rows, int cols, int Mp, int Kp,
+                            int batch, hipStream_t stream) {
     dim3 grid((Mp / 64) * (Kp / 64), batch), block(256);
-    hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, partials, nparts, X, XT, strideX, rows,
-                       cols, Mp, Kp);
+    hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, partials, nparts, X, ldx, strideX, XT, ldxt,
+                       strideXT, rows, cols, Mp, Kp);
     return hipGetLastError();
 }
 

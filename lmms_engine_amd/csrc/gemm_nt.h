@@ -11,7 +11,12 @@ enum {
     GEMM_CFG_128x128_W4_DLDS = 3,
     GEMM_CFG_256x256_W4_DLDS = 4,
     GEMM_CFG_256x256_W8_DLDS = 5,
-    GEMM_CFG_COUNT = 6
+    GEMM_CFG_128x128_W4_PIPE = 6,
+    GEMM_CFG_256x256_W4_PIPE = 7,
+    GEMM_CFG_256x256_W8_PIPE = 8,
+    GEMM_CFG_128x128_W4_PIPE4 = 9,
+    GEMM_CFG_256x256_W4_PIPE4 = 10,
+    GEMM_CFG_COUNT = 11
 };
 
 struct GemmArgs {

@@ -130,6 +130,89 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
     }
 }
 
+// The same epilogue staged through LDS (free once the main loop is over) so that global
+// traffic is 16-byte vectors: the tile is kept as Tt[n][m] (n = local column, m = local row of
+// the accumulator tile), row stride BM*2+16 bytes.  The elementwise source Et has exactly that
+// orientation, so it is loaded into Tt with coalesced reads, each lane then replaces its own
+// 8-byte pieces by the rounded results, and the tile leaves as rows of Ct (straight) and rows
+// of C (gathered down the columns of Tt).  Diagonal tiles of the symmetric kernels write the
+// full tile once: acc(i,j) and acc(j,i) are sums of the same exact products in the same order.
+template <int BM, int BN>
+constexpr int epilogue_lds_bytes() { return BN * (BM * 2 + 16); }
+
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__device__ __forceinline__ void epilogue_lds(const GemmArgs& g, const TileCoord& tc,
+                                             f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], unsigned char* smem) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int S = BM * 2 + 16;
+    constexpr int CPR = BM / 8;  // 16-byte chunks per Tt row
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN, hi = lane >> 5;
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+    const bool diag = (EPI != EPI_BX) && (tc.ti == tc.tj);
+    bf16_t* C = g.C ? g.C + tc.bidx * g.strideC : nullptr;
+    bf16_t* Ct = g.Ct ? g.Ct + tc.bidx * g.strideCt : nullptr;
+    __syncthreads();  // every wave is done reading the operand stages
+    if (EPI != EPI_SYRK) {
+        const bf16_t* Et = g.Et + tc.bidx * g.strideEt + n0 * g.ldet + m0;
+#pragma unroll 4
+        for (int c = tid; c < BN * CPR; c += NT) {
+            const int n = c / CPR, k = c % CPR;
+            *(u32x4*)(smem + n * S + k * 16) = *(const u32x4*)(Et + (long)n * g.ldet + k * 8);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int n = wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int m = wm * WTM + i * 32 + q * 8 + hi * 4;
+                unsigned char* p = smem + n * S + m * 2;
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = rbf(acc[i][j][q * 4 + r]);
+                if (EPI != EPI_SYRK) {
+                    const bf16x4 e = *(const bf16x4*)p;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (EPI == EPI_SYMPOLY) v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + rbf(g.s1 * v[r]));
+                        else v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + v[r]);
+                    }
+                }
+                bf16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[r] = f2bf(v[r]);
+                *(bf16x4*)p = o;
+            }
+        }
+    }
+    __syncthreads();
+    if (Ct) {
+        bf16_t* dst = Ct + n0 * g.ldct + m0;
+#pragma unroll 4
+        for (int c = tid; c < BN * CPR; c += NT) {
+            const int n = c / CPR, k = c % CPR;
+            *(u32x4*)(dst + (long)n * g.ldct + k * 8) = *(const u32x4*)(smem + n * S + k * 16);
+        }
+    }
+    if (C && !diag) {
+        bf16_t* dst = C + m0 * g.ldc + n0;
+#pragma unroll 2
+        for (int idx = tid; idx < BM * (BN / 8); idx += NT) {
+            const int m = idx % BM, c = idx / BM;  // consecutive lanes walk down a column of C
+            bf16x8 o;
+#pragma unroll
+            for (int r = 0; r < 8; ++r) o[r] = *(const bf16_t*)(smem + (c * 8 + r) * S + m * 2);
+            *(bf16x8*)(dst + (long)m * g.ldc + c * 8) = o;
+        }
+    }
+}
+
 // ---- variant 1: global -> registers -> LDS, two LDS stages, one barrier per k-tile -------
 template <int BM, int BN, int WGM, int WGN, int EPI>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g) {
@@ -215,8 +298,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g
     float ssum = 0.f;
     for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
     if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
-#else
+#elif defined(EXP_DIRECT_EPI)
     epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc);
+#else
+    epilogue_lds<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
@@ -360,16 +445,354 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_dlds_kernel(const GemmA
     float ssum = 0.f;
     for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
     if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
-#else
+#elif defined(EXP_DIRECT_EPI)
     epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc);
+#else
+    epilogue_lds<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
-template <int BM, int BN, int WGM, int WGN, int EPI, bool DLDS>
+// ---- variant 3: direct global -> LDS feed, software pipelined, one barrier per k-tile -----
+// Per k-tile a wave issues FM*FN*4 MFMAs, (FM+FN)*4 LDS fragment reads and LA+LB 1 KB loads.
+// Every non-MFMA instruction is placed between two MFMAs so that it issues in their shadow:
+//   k-steps 0..2 : MFMAs of step s interleaved with the fragment reads of step s+1;
+//   k-step 3     : the wave has now read everything it needs from this stage, so it waits
+//                  for its own loads of the next k-tile, crosses the one barrier, and then
+//                  interleaves the last MFMAs with the loads of k-tile t+2 (into the stage just
+//                  released) and with the fragment reads of step 0 of k-tile t+1.
+// The fences (sched_barrier) pin that order; without them the scheduler sinks every LDS read
+// next to its first use and the MFMA pipe idles for an LDS round trip per k-step.
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmArgs g) {
+    constexpr int NW = WGM * WGN;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE = A_BYTES + B_BYTES;
+    constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;
+    constexpr int KS = BK / 16;
+    constexpr int NMF = FM * FN, NRD = FM + FN, NLD = LA + LB;
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "dma split");
+    static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const TileCoord tc = decode_tile<EPI>(g);
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+#ifdef EXP_SAME_TILE
+    const bf16_t* Pb = g.P;
+    const bf16_t* Qb = g.Q;
+#else
+    const bf16_t* Pb = g.P + tc.bidx * g.strideP + m0 * g.ldp;
+    const bf16_t* Qb = g.Q + tc.bidx * g.strideQ + n0 * g.ldq;
+#endif
+
+    const int drow = lane >> 3;
+    const bf16_t* pa = Pb + (long)(wave * 8 * LA + drow) * g.ldp;
+    const bf16_t* pb = Qb + (long)(wave * 8 * LB + drow) * g.ldq;
+    const int lds_a = wave * 8 * LA * ROW_BYTES;
+    const int lds_b = A_BYTES + wave * 8 * LB * ROW_BYTES;
+    const int ch_even = ((lane & 7) ^ (drow >> 1)) * 8, ch_odd = ((lane & 7) ^ (4 | (drow >> 1))) * 8;
+
+    // load instruction n (0..NLD-1) of a k-tile: A rows first, then B rows
+    auto issue_one = [&](int n, int stage, int k0) {
+        unsigned char* s = smem + stage * STAGE;
+        if (n < LA) {
+            const int ch = ((wave * LA + n) & 1) ? ch_odd : ch_even;
+            __builtin_amdgcn_global_load_lds((glb_void_ptr)(pa + (long)n * 8 * g.ldp + k0 + ch),
+                                             (lds_void_ptr)(s + lds_a + n * 8 * ROW_BYTES), 16, 0, 0);
+        } else {
+            const int i = n - LA;
+            const int ch = ((wave * LB + i) & 1) ? ch_odd : ch_even;
+            __builtin_amdgcn_global_load_lds((glb_void_ptr)(pb + (long)i * 8 * g.ldq + k0 + ch),
+                                             (lds_void_ptr)(s + lds_b + i * 8 * ROW_BYTES), 16, 0, 0);
+        }
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int sw = (lane >> 1) & 7, hi = lane >> 5;
+    const int a_off = (wm * WTM + (lane & 31)) * ROW_BYTES;
+    const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROW_BYTES;
+
+    bf16x8 fr[2][NRD];  // fragment double buffer: [0..FM) rows of P, [FM..NRD) rows of Q
+    auto read_one = [&](int buf, int n, const unsigned char* st, int ks) {
+        const int co = (((ks << 1) | hi) ^ sw) << 4;
+        if (n < FM) fr[buf][n] = *(const bf16x8*)(st + a_off + n * 32 * ROW_BYTES + co);
+        else fr[buf][n] = *(const bf16x8*)(st + b_off + (n - FM) * 32 * ROW_BYTES + co);
+    };
+    auto mfma_one = [&](int buf, int idx) {
+        const int i = idx / FN, j = idx % FN;
+#ifdef EXP_NO_MFMA
+        acc[i][j][0] += (float)fr[buf][i][0] * (float)fr[buf][FM + j][0];
+#else
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[buf][i], fr[buf][FM + j], acc[i][j], 0, 0, 0);
+#endif
+    };
+
+    const int nk = g.kdim / BK;
+#pragma unroll
+    for (int n = 0; n < NLD; ++n) issue_one(n, 0, 0);
+    if (nk > 1) {
+#pragma unroll
+        for (int n = 0; n < NLD; ++n) issue_one(n, 1, BK);
+        WAIT_VM(NLD);
+    } else {
+        WAIT_VM(0);
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < NRD; ++n) read_one(0, n, smem, 0);
+
+#ifdef EXP_TRACE
+    long long* trace = (long long*)g.Ct + (long)blockIdx.x * 4096 + (threadIdx.x >> 6) * 1024;
+    int tn = 0;
+#define TRACE_POINT() do { if (lane == 0 && tn < 1000) trace[tn] = clock64(); ++tn; } while (0)
+#else
+#define TRACE_POINT() do {} while (0)
+#endif
+    for (int kt = 0; kt < nk; ++kt) {
+        const unsigned char* st = smem + (kt & 1) * STAGE;
+        const unsigned char* stn = smem + ((kt + 1) & 1) * STAGE;
+        TRACE_POINT();
+#pragma unroll
+        for (int ks = 0; ks < KS - 1; ++ks) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int idx = 0; idx < NMF; ++idx) {
+                mfma_one(ks & 1, idx);
+                if (idx < NRD) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    read_one((ks + 1) & 1, idx, st, ks + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // Fragments of the last k-step are in: this wave is done with stage kt&1.  The tail is
+        // branch free: past the end it re-loads the last k-tile into a stage nobody reads and
+        // pre-reads fragments nobody uses, which costs 2 of nk loads and keeps the MFMAs in
+        // one basic block.
+        TRACE_POINT();
+        WAIT_LGKM0();
+        WAIT_VM(0);  // its loads of k-tile kt+1 (the only ones in flight) have landed
+        TRACE_POINT();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        TRACE_POINT();
+        const int k2 = (kt + 2 < nk ? kt + 2 : nk - 1) * BK;
+        constexpr int PER = (NLD + NRD + NMF - 1) / NMF;  // loads and reads per MFMA slot
+#pragma unroll
+        for (int idx = 0; idx < NMF; ++idx) {
+            mfma_one((KS - 1) & 1, idx);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < PER; ++u) {
+                const int o = idx * PER + u;
+                if (o < NRD) read_one(KS & 1, o, stn, 0);
+                else if (o < NRD + NLD) issue_one(o - NRD, kt & 1, k2);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    WAIT_VM(0);  // the dummy loads of the last two tails must not land in the epilogue's tile
+#ifdef EXP_NO_EPI
+    float ssum = 0.f;
+    for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
+    if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
+#else
+    epilogue_lds<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+#endif
+}
+
+// ---- variant 4: 32-wide k-tiles in four LDS stages ----------------------------------------
+// The L1 -> LDS path moves 64 B/clk per CU, so feeding a 256x256 tile keeps it busy half of
+// the time; when the loads of a k-tile are issued in one burst (variant 3, two stages) every
+// wave of the CU queues on the one address path and its MFMAs starve behind the blocked
+// load.  Four stages of 32 columns leave a stage free for a whole k-tile, so the loads are
+// spread evenly: 4 per 16 MFMAs.  Timeline of wave w for k-tile t (stage t&3, two k-steps):
+//   phase A: MFMAs of k-step 0 | fragment reads of k-step 1 | B-half loads of k-tile t+3
+//   wait own reads; wait own loads of k-tile t+1; barrier   (stage t&3 is now free)
+//   phase B: MFMAs of k-step 1 | fragment reads of k-tile t+1 step 0 | A-half loads of k-tile t+4
+// LDS rows are 64 B (4 chunks); chunk c of row r sits at position c ^ ((r>>2)&3).
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe4_kernel(const GemmArgs g) {
+    constexpr int NW = WGM * WGN;
+    constexpr int BK4 = 32, ROWB = 64, NST = 4;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int LA = BM / 16 / NW, LB = BN / 16 / NW;  // 1 KB loads (16 rows) per wave per k-tile
+    constexpr int NMF = FM * FN, NRD = FM + FN;
+    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "dma split");
+    // Slot plan of one phase (NMF MFMAs, NRD fragment reads, L loads): the loads sit behind every
+    // (NMF/L)-th MFMA so that the four waves of the CU, which run in lockstep, hand the one L1
+    // address path 4 loads (64 cycles of work) per NMF/L MFMAs instead of 16 back to back; the
+    // reads fill the other slots from the front.
+    constexpr int LSP_A = NMF / LB > 0 ? NMF / LB : 1, LSP_B = NMF / LA > 0 ? NMF / LA : 1;
+    constexpr int RPS_A = (NRD + (NMF - NMF / LSP_A) - 1) / (NMF - NMF / LSP_A > 0 ? NMF - NMF / LSP_A : 1);
+    constexpr int RPS_B = (NRD + (NMF - NMF / LSP_B) - 1) / (NMF - NMF / LSP_B > 0 ? NMF - NMF / LSP_B : 1);
+    static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const TileCoord tc = decode_tile<EPI>(g);
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+    const bf16_t* Pb = g.P + tc.bidx * g.strideP + m0 * g.ldp;
+    const bf16_t* Qb = g.Q + tc.bidx * g.strideQ + n0 * g.ldq;
+
+    // lane L of a load lands on row L>>2, position L&3 and so fetches chunk (L&3)^((L>>4)&3)
+    const int drow = lane >> 2;
+    const int dch = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;
+    const bf16_t* pa = Pb + (long)(wave * 16 * LA + drow) * g.ldp + dch;
+    const bf16_t* pb = Qb + (long)(wave * 16 * LB + drow) * g.ldq + dch;
+    const int lds_a = wave * 16 * LA * ROWB;
+    const int lds_b = A_BYTES + wave * 16 * LB * ROWB;
+    const int nk = g.kdim / BK4;
+
+    auto issue_a = [&](int n, int kt) {  // kt may run past the end: re-load the last k-tile
+        const int kk = (kt < nk ? kt : nk - 1) * BK4;
+        __builtin_amdgcn_global_load_lds((glb_void_ptr)(pa + (long)n * 16 * g.ldp + kk),
+                                         (lds_void_ptr)(smem + (kt & 3) * STAGE + lds_a + n * 16 * ROWB), 16, 0, 0);
+    };
+    auto issue_b = [&](int n, int kt) {
+        const int kk = (kt < nk ? kt : nk - 1) * BK4;
+        __builtin_amdgcn_global_load_lds((glb_void_ptr)(pb + (long)n * 16 * g.ldq + kk),
+                                         (lds_void_ptr)(smem + (kt & 3) * STAGE + lds_b + n * 16 * ROWB), 16, 0, 0);
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int sw = (lane >> 2) & 3, hi = lane >> 5;
+    const int a_off = (wm * WTM + (lane & 31)) * ROWB;
+    const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROWB;
+
+    bf16x8 fr[2][NRD];
+    auto read_one = [&](int buf, int n, const unsigned char* st, int ks) {
+        const int co = (((ks << 1) | hi) ^ sw) << 4;
+        if (n < FM) fr[buf][n] = *(const bf16x8*)(st + a_off + n * 32 * ROWB + co);
+        else fr[buf][n] = *(const bf16x8*)(st + b_off + (n - FM) * 32 * ROWB + co);
+    };
+    auto mfma_one = [&](int buf, int idx) {
+        const int i = idx / FN, j = idx % FN;
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[buf][i], fr[buf][FM + j], acc[i][j], 0, 0, 0);
+    };
+
+    // prologue: k-tiles 0..2 and the A half of k-tile 3
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+#pragma unroll
+        for (int n = 0; n < LA; ++n) issue_a(n, t);
+#pragma unroll
+        for (int n = 0; n < LB; ++n) issue_b(n, t);
+    }
+#pragma unroll
+    for (int n = 0; n < LA; ++n) issue_a(n, 3);
+    WAIT_VM(2 * (LA + LB) + LA);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < NRD; ++n) read_one(0, n, smem, 0);
+
+#ifdef EXP_TRACE
+    long long* trace = (long long*)g.Ct + (long)blockIdx.x * 4096 + (threadIdx.x >> 6) * 1024;
+    int tn = 0;
+#endif
+    for (int kt = 0; kt < nk; ++kt) {
+        const unsigned char* st = smem + (kt & 3) * STAGE;
+        const unsigned char* stn = smem + ((kt + 1) & 3) * STAGE;
+        TRACE_POINT();
+        // phase A
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int idx = 0; idx < NMF; ++idx) {
+            mfma_one(0, idx);
+            __builtin_amdgcn_sched_barrier(0);
+            if ((idx + 1) % LSP_A == 0) {
+#ifndef EXP4_NO_DMA
+                if (idx / LSP_A < LB) issue_b(idx / LSP_A, kt + 3);
+#endif
+            } else {
+#ifndef EXP4_NO_RD
+                const int r0 = (idx - idx / LSP_A) * RPS_A;
+#pragma unroll
+                for (int u = 0; u < RPS_A; ++u)
+                    if (r0 + u < NRD) read_one(1, r0 + u, st, 1);
+#endif
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // own reads of this stage are complete, own loads of k-tile kt+1 have landed
+        TRACE_POINT();
+        WAIT_LGKM0();
+#ifndef EXP4_NO_DMA
+        WAIT_VM(2 * (LA + LB));
+#endif
+        TRACE_POINT();
+        asm volatile("" ::: "memory");
+#ifndef EXP4_NO_BAR
+        __builtin_amdgcn_s_barrier();
+#endif
+        asm volatile("" ::: "memory");
+        TRACE_POINT();
+        // phase B
+#pragma unroll
+        for (int idx = 0; idx < NMF; ++idx) {
+            mfma_one(1, idx);
+            __builtin_amdgcn_sched_barrier(0);
+            if ((idx + 1) % LSP_B == 0) {
+#ifndef EXP4_NO_DMA
+                if (idx / LSP_B < LA) issue_a(idx / LSP_B, kt + 4);
+#endif
+            } else {
+#ifndef EXP4_NO_RD
+                const int r0 = (idx - idx / LSP_B) * RPS_B;
+#pragma unroll
+                for (int u = 0; u < RPS_B; ++u)
+                    if (r0 + u < NRD) read_one(0, r0 + u, stn, 0);
+#endif
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
+#ifdef EXP_NO_EPI
+    float ssum = 0.f;
+    for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
+    if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
+#else
+    epilogue_lds<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+#endif
+}
+
+template <int BM, int BN, int WGM, int WGN, int EPI, int FEED>
 hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
-    constexpr int smem = 2 * (BM + BN) * ROW_BYTES;
+    constexpr int stage2 = 2 * (BM + BN) * ROW_BYTES, epi = epilogue_lds_bytes<BM, BN>();
+    constexpr int smem = stage2 > epi ? stage2 : epi;
     static bool configured = false;  // per instantiation; the attribute is idempotent
-    auto kern = DLDS ? gemm_nt_dlds_kernel<BM, BN, WGM, WGN, EPI> : gemm_nt_kernel<BM, BN, WGM, WGN, EPI>;
+    auto kern = FEED == 3 ? gemm_nt_pipe4_kernel<BM, BN, WGM, WGN, EPI>
+              : FEED == 2 ? gemm_nt_pipe_kernel<BM, BN, WGM, WGN, EPI>
+              : FEED == 1 ? gemm_nt_dlds_kernel<BM, BN, WGM, WGN, EPI>
+                          : gemm_nt_kernel<BM, BN, WGM, WGN, EPI>;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
@@ -382,12 +805,17 @@ hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
 template <int EPI>
 hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t stream) {
     switch (cfg) {
-        case GEMM_CFG_128x128_W4: return launch_one<128, 128, 2, 2, EPI, false>(g, nblocks, stream);
-        case GEMM_CFG_256x256_W4: return launch_one<256, 256, 2, 2, EPI, false>(g, nblocks, stream);
-        case GEMM_CFG_256x256_W8: return launch_one<256, 256, 2, 4, EPI, false>(g, nblocks, stream);
-        case GEMM_CFG_128x128_W4_DLDS: return launch_one<128, 128, 2, 2, EPI, true>(g, nblocks, stream);
-        case GEMM_CFG_256x256_W4_DLDS: return launch_one<256, 256, 2, 2, EPI, true>(g, nblocks, stream);
-        case GEMM_CFG_256x256_W8_DLDS: return launch_one<256, 256, 2, 4, EPI, true>(g, nblocks, stream);
+        case GEMM_CFG_128x128_W4: return launch_one<128, 128, 2, 2, EPI, 0>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W4: return launch_one<256, 256, 2, 2, EPI, 0>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8: return launch_one<256, 256, 2, 4, EPI, 0>(g, nblocks, stream);
+        case GEMM_CFG_128x128_W4_DLDS: return launch_one<128, 128, 2, 2, EPI, 1>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W4_DLDS: return launch_one<256, 256, 2, 2, EPI, 1>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8_DLDS: return launch_one<256, 256, 2, 4, EPI, 1>(g, nblocks, stream);
+        case GEMM_CFG_128x128_W4_PIPE: return launch_one<128, 128, 2, 2, EPI, 2>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W4_PIPE: return launch_one<256, 256, 2, 2, EPI, 2>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8_PIPE: return launch_one<256, 256, 2, 4, EPI, 2>(g, nblocks, stream);
+        case GEMM_CFG_128x128_W4_PIPE4: return launch_one<128, 128, 2, 2, EPI, 3>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W4_PIPE4: return launch_one<256, 256, 2, 2, EPI, 3>(g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -397,11 +825,16 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
 int gemm_cfg_tile(int cfg) {
     switch (cfg) {
         case GEMM_CFG_128x128_W4:
-        case GEMM_CFG_128x128_W4_DLDS: return 128;
+        case GEMM_CFG_128x128_W4_DLDS:
+        case GEMM_CFG_128x128_W4_PIPE:
+        case GEMM_CFG_128x128_W4_PIPE4: return 128;
         case GEMM_CFG_256x256_W4:
         case GEMM_CFG_256x256_W8:
         case GEMM_CFG_256x256_W4_DLDS:
-        case GEMM_CFG_256x256_W8_DLDS: return 256;
+        case GEMM_CFG_256x256_W8_DLDS:
+        case GEMM_CFG_256x256_W4_PIPE:
+        case GEMM_CFG_256x256_W8_PIPE:
+        case GEMM_CFG_256x256_W4_PIPE4: return 256;
         default: return 0;
     }
 }

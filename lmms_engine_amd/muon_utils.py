@@ -84,21 +84,17 @@ def matmul_transpose_assign(d_in: Tensor, d_out: Tensor) -> None:
     geo = _abi.geometry(M, max(K, M))  # tile choice follows the small side
     tile = geo["tile"]
     Mp, Kp = -(-M // tile) * tile, -(-K // tile) * tile
+    ldx, lda = Kp + 128, Mp + 128  # padded pitches keep the rows of a tile on different L2 channels
     with torch.cuda.device(d_in.device):
-        if (Mp, Kp) == (M, K) and d_in.is_contiguous():
-            x = d_in
-        else:
-            x = torch.zeros(Mp, Kp, dtype=torch.bfloat16, device=d_in.device)
-            x[:M, :K].copy_(d_in)
-        direct = Mp == M and d_out.is_contiguous()
-        a = d_out if direct else torch.empty(Mp, Mp, dtype=torch.bfloat16, device=d_in.device)
+        x = torch.zeros(Mp, ldx, dtype=torch.bfloat16, device=d_in.device)
+        x[:M, :K].copy_(d_in)
+        a = torch.empty(Mp, lda, dtype=torch.bfloat16, device=d_in.device)
         _abi.check(
-            _abi.lib().muon_hip_syrk_bf16(x.data_ptr(), a.data_ptr(), Mp, Kp, 1, _abi.CFG_AUTO,
+            _abi.lib().muon_hip_syrk_bf16(x.data_ptr(), ldx, a.data_ptr(), lda, Mp, Kp, 1, _abi.CFG_AUTO,
                                           _abi.stream_ptr(d_in.device)),
             "syrk",
         )
-        if not direct:
-            d_out.copy_(a[:M, :M])
+        d_out.copy_(a[:M, :M])
 
 
 def matmul_transpose(d_in: Tensor) -> Tensor:

@@ -47,7 +47,7 @@ def _assert_product_close(got, ref64, absprod):
     assert not bad.any(), f"{int(bad.sum())} elements outside one bf16 ulp"
 
 
-CFGS = [0, 1, 2, 3, 4, 5]
+CFGS = list(range(11))
 
 
 @pytest.mark.parametrize("cfg", CFGS)
@@ -58,7 +58,7 @@ def test_syrk_matches_fp64_and_is_symmetric(env, cfg, M, K, batch):
     X = torch.randn(batch, M, K, generator=g).bfloat16()
     Xd = X.to(env["dev"])
     A = torch.full((batch, M, M), float("nan"), dtype=torch.bfloat16, device=env["dev"])
-    env["abi"].check(env["lib"].muon_hip_syrk_bf16(Xd.data_ptr(), A.data_ptr(), M, K, batch, cfg, 0))
+    env["abi"].check(env["lib"].muon_hip_syrk_bf16(Xd.data_ptr(), K, A.data_ptr(), M, M, K, batch, cfg, 0))
     torch.cuda.synchronize()
     A = A.cpu()
     assert torch.equal(A, A.mT), "X·Xᵀ must be symmetric bit for bit"
@@ -78,7 +78,7 @@ def test_sympoly_rounding_points(env, cfg):
     Ad = A.to(env["dev"])
     B = torch.full_like(Ad, float("nan"))
     a, b, c = O.NS_COEFFS
-    env["abi"].check(env["lib"].muon_hip_sympoly_bf16(Ad.data_ptr(), B.data_ptr(), M, batch, b, c, cfg, 0))
+    env["abi"].check(env["lib"].muon_hip_sympoly_bf16(Ad.data_ptr(), B.data_ptr(), M, M, batch, b, c, cfg, 0))
     torch.cuda.synchronize()
     B = B.cpu()
     assert torch.equal(B, B.mT)
@@ -107,7 +107,7 @@ def test_bx_axpy_rounding_points(env, cfg, outputs):
     XT = X.mT.contiguous().to(dev)
     a = O.NS_COEFFS[0]
     env["abi"].check(env["lib"].muon_hip_bx_axpy_bf16(
-        Bm.to(dev).data_ptr(), XT.data_ptr(), Xo.data_ptr() if outputs != "xt" else None,
+        Bm.to(dev).data_ptr(), M, XT.data_ptr(), M, Xo.data_ptr() if outputs != "xt" else None, K,
         XTo.data_ptr() if outputs != "x" else None, M, K, batch, a, cfg, 0))
     torch.cuda.synchronize()
     for i in range(batch):
@@ -127,12 +127,13 @@ def test_bx_axpy_rounding_points(env, cfg, outputs):
 def test_gemm_entry_points_reject_bad_shapes(env):
     lib, abi = env["lib"], env["abi"]
     x = torch.zeros(256, 256, dtype=torch.bfloat16, device=env["dev"])
-    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 200, 256, 1, 0, 0) == -2
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), 256, x.data_ptr(), 256, 200, 256, 1, 0, 0) == -2
     assert b"multiples" in lib.muon_hip_last_error()
-    assert lib.muon_hip_syrk_bf16(None, x.data_ptr(), 256, 256, 1, 0, 0) == -1
-    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 256, 256, 1, 99, 0) == -1
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), 128, x.data_ptr(), 256, 256, 256, 1, 0, 0) == -2  # pitch < width
+    assert lib.muon_hip_syrk_bf16(None, 256, x.data_ptr(), 256, 256, 256, 1, 0, 0) == -1
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), 256, x.data_ptr(), 256, 256, 256, 1, 99, 0) == -1
     with pytest.raises(abi.MuonHipError):
-        abi.check(lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), None, None, 256, 256, 1, 1.0, 0, 0))
+        abi.check(lib.muon_hip_bx_axpy_bf16(x.data_ptr(), 256, x.data_ptr(), 256, None, 256, None, 256, 256, 1, 1.0, 0, 0))
 
 
 NS_SHAPES = [(64, 160), (160, 64), (33, 47), (100, 300), (300, 100), (128, 896), (896, 128), (256, 256), (512, 1024)]
