@@ -38,6 +38,7 @@ struct GemmArgs {
     long strideEt;
     int ldet;
     float s0, s1;  // SYMPOLY: (b, c); BX: (a, -)
+    int stagger;   // cycles by which XCD x delays its first tile (x * stagger); 0 = off
 };
 
 int gemm_cfg_tile(int cfg);

@@ -64,8 +64,21 @@ struct TileCoord {
     int bidx, ti, tj;
 };
 
+// Every tile takes the same time, so without help all CUs reach their epilogues together and
+// the write-back arrives at HBM as one burst per round while the MFMAs idle.  Delaying the
+// first tile of XCD x by x/8 of a tile time keeps the eight XCDs out of phase for the rest of
+// the launch, so each XCD's burst drains while the others compute.
+__device__ __forceinline__ void stagger_first_round(const GemmArgs& g) {
+    if (g.stagger > 0 && blockIdx.x < 256) {
+        const long long wait = (long long)(blockIdx.x % XCD_COUNT) * g.stagger;
+        const long long t0 = clock64();
+        while (clock64() - t0 < wait) __builtin_amdgcn_s_sleep(32);
+    }
+}
+
 template <int EPI>
 __device__ __forceinline__ TileCoord decode_tile(const GemmArgs& g) {
+    stagger_first_round(g);
     const int logical = xcd_remap(blockIdx.x, gridDim.x);
     TileCoord tc;
     tc.bidx = logical / g.tiles_per_mat;
@@ -140,6 +153,13 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
 template <int BM, int BN>
 constexpr int epilogue_lds_bytes() { return BN * (BM * 2 + 16); }
 
+#ifdef EXP_TRACE_EPI
+__device__ long long* g_epi_trace;
+#define EPI_POINT(n) do { if (threadIdx.x == 0) g_epi_trace[(long)blockIdx.x * 8 + (n)] = clock64(); } while (0)
+#else
+#define EPI_POINT(n) do {} while (0)
+#endif
+
 template <int BM, int BN, int WGM, int WGN, int EPI>
 __device__ __forceinline__ void epilogue_lds(const GemmArgs& g, const TileCoord& tc,
                                              f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], unsigned char* smem) {
@@ -154,7 +174,9 @@ __device__ __forceinline__ void epilogue_lds(const GemmArgs& g, const TileCoord&
     const bool diag = (EPI != EPI_BX) && (tc.ti == tc.tj);
     bf16_t* C = g.C ? g.C + tc.bidx * g.strideC : nullptr;
     bf16_t* Ct = g.Ct ? g.Ct + tc.bidx * g.strideCt : nullptr;
+    EPI_POINT(0);
     __syncthreads();  // every wave is done reading the operand stages
+    EPI_POINT(1);
     if (EPI != EPI_SYRK) {
         const bf16_t* Et = g.Et + tc.bidx * g.strideEt + n0 * g.ldet + m0;
 #pragma unroll 4
@@ -164,6 +186,7 @@ __device__ __forceinline__ void epilogue_lds(const GemmArgs& g, const TileCoord&
         }
         __syncthreads();
     }
+    EPI_POINT(2);
 #pragma unroll
     for (int i = 0; i < FM; ++i) {
 #pragma unroll
@@ -191,7 +214,9 @@ __device__ __forceinline__ void epilogue_lds(const GemmArgs& g, const TileCoord&
             }
         }
     }
+    EPI_POINT(3);
     __syncthreads();
+    EPI_POINT(4);
     if (Ct) {
         bf16_t* dst = Ct + n0 * g.ldct + m0;
 #pragma unroll 4
@@ -200,6 +225,7 @@ __device__ __forceinline__ void epilogue_lds(const GemmArgs& g, const TileCoord&
             *(u32x4*)(dst + (long)n * g.ldct + k * 8) = *(const u32x4*)(smem + n * S + k * 16);
         }
     }
+    EPI_POINT(5);
     if (C && !diag) {
         bf16_t* dst = C + m0 * g.ldc + n0;
 #pragma unroll 2
@@ -210,6 +236,142 @@ __device__ __forceinline__ void epilogue_lds(const GemmArgs& g, const TileCoord&
             for (int r = 0; r < 8; ++r) o[r] = *(const bf16_t*)(smem + (c * 8 + r) * S + m * 2);
             *(bf16x8*)(dst + (long)m * g.ldc + c * 8) = o;
         }
+    }
+    EPI_POINT(6);
+#ifdef EXP_TRACE_EPI
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    EPI_POINT(7);
+#endif
+}
+
+// Epilogue with both output orientations coalesced.  Stage 1 (all waves): the elementwise
+// source Et comes through LDS as Et[n][m] with 16-byte loads, each lane picks its 8-byte pieces
+// and keeps the rounded results of all its fragments in registers.  Stage 2, one half of the
+// columns at a time (LDS cannot hold both orientations of a whole tile): the owners drop their
+// items into Tt[n][m] (the orientation of Ct) and T[m][n] (the orientation of C), and
+// everybody copies whole rows out with 16-byte stores.
+template <int BM, int BN>
+constexpr int epilogue_lds2_bytes() {
+    constexpr int halves = (BN / 2) * (BM * 2 + 16) + BM * (BN + 16), whole = BN * (BM * 2 + 16);
+    return halves > whole ? halves : whole;
+}
+
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__device__ __forceinline__ void epilogue_lds2(const GemmArgs& g, const TileCoord& tc,
+                                              f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], unsigned char* smem) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int HN = BN / 2;             // columns per half
+    constexpr int S1 = BM * 2 + 16;        // Tt row pitch (bytes)
+    constexpr int S2 = HN * 2 + 16;        // T row pitch (bytes)
+    constexpr int T_OFF = HN * S1;
+    constexpr int CPR1 = BM / 8, CPR2 = HN / 8;  // 16-byte chunks per row
+    constexpr int NL1 = HN * CPR1 / NT, NL2 = BM * CPR2 / NT;
+    static_assert(WTN <= HN && HN % WTN == 0, "a wave's columns lie in one half");
+    static_assert((HN * CPR1) % NT == 0 && (BM * CPR2) % NT == 0, "row copies divide evenly");
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN, hi = lane >> 5;
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+    const bool diag = (EPI != EPI_BX) && (tc.ti == tc.tj);
+    bf16_t* C = (g.C && !diag) ? g.C + tc.bidx * g.strideC + m0 * g.ldc + n0 : nullptr;
+    bf16_t* Ct = g.Ct ? g.Ct + tc.bidx * g.strideCt + n0 * g.ldct + m0 : nullptr;
+    unsigned char* Tt = smem;
+    unsigned char* T = smem + T_OFF;
+
+    // Stage 1, every wave at once: results of all fragments, rounded, packed 4 rows per item.
+    bf16x4 res[FM][FN][4];
+    EPI_POINT(0);
+    __syncthreads();  // the operand stages are no longer read
+    EPI_POINT(1);
+    if (EPI != EPI_SYRK) {
+        // the whole Et tile goes through LDS as Et[n][m] (pitch S1) with coalesced 16-byte loads
+        const bf16_t* Et = g.Et + tc.bidx * g.strideEt + n0 * g.ldet + m0;
+        constexpr int NLE = BN * CPR1 / NT;
+#pragma unroll
+        for (int b = 0; b < NLE; b += 16) {
+            u32x4 ev[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int c = tid + (b + u) * NT, n = c / CPR1, k = c % CPR1;
+                if (b + u < NLE) ev[u] = *(const u32x4*)(Et + (long)n * g.ldet + k * 8);
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int c = tid + (b + u) * NT, n = c / CPR1, k = c % CPR1;
+                if (b + u < NLE) *(u32x4*)(smem + n * S1 + k * 16) = ev[u];
+            }
+        }
+        __syncthreads();
+    }
+    EPI_POINT(2);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const int n = wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int m = wm * WTM + i * 32 + q * 8 + hi * 4;
+                float v[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) v[r] = rbf(acc[i][j][q * 4 + r]);
+                if (EPI != EPI_SYRK) {
+                    const bf16x4 e = *(const bf16x4*)(smem + n * S1 + m * 2);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (EPI == EPI_SYMPOLY) v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + rbf(g.s1 * v[r]));
+                        else v[r] = rbf(rbf(g.s0 * bf2f(e[r])) + v[r]);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) res[i][j][q][r] = f2bf(v[r]);
+            }
+        }
+    }
+    EPI_POINT(3);
+    // Stage 2, one half of the columns at a time: owners drop their items into Tt and T, then
+    // everybody copies whole rows out.
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        __syncthreads();  // Et tile (h == 0) or the previous half (h == 1) is no longer read
+        if ((wn * WTN) / HN == h) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i) {
+#pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    const int n = (wn * WTN) % HN + j * 32 + (lane & 31);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int m = wm * WTM + i * 32 + q * 8 + hi * 4;
+                        if (Ct) *(bf16x4*)(Tt + n * S1 + m * 2) = res[i][j][q];
+                        if (C) {
+#pragma unroll
+                            for (int r = 0; r < 4; ++r) *(bf16_t*)(T + (m + r) * S2 + n * 2) = res[i][j][q][r];
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        if (h == 0) EPI_POINT(4);
+        if (Ct) {
+#pragma unroll
+            for (int u = 0; u < NL1; ++u) {
+                const int c = tid + u * NT, n = c / CPR1, k = c % CPR1;
+                *(u32x4*)(Ct + (long)(h * HN + n) * g.ldct + k * 8) = *(const u32x4*)(Tt + n * S1 + k * 16);
+            }
+        }
+        if (h == 0) EPI_POINT(5);
+        if (C) {
+#pragma unroll
+            for (int u = 0; u < NL2; ++u) {
+                const int c = tid + u * NT, m = c / CPR2, k = c % CPR2;
+                *(u32x4*)(C + (long)m * g.ldc + h * HN + k * 8) = *(const u32x4*)(T + m * S2 + k * 16);
+            }
+        }
+        if (h == 0) EPI_POINT(6);
+        if (h == 1) EPI_POINT(7);
     }
 }
 
@@ -301,7 +463,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g
 #elif defined(EXP_DIRECT_EPI)
     epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc);
 #else
-    epilogue_lds<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
@@ -448,7 +610,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_dlds_kernel(const GemmA
 #elif defined(EXP_DIRECT_EPI)
     epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc);
 #else
-    epilogue_lds<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
@@ -611,7 +773,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
     if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
 #else
-    epilogue_lds<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
@@ -780,13 +942,13 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe4_kernel(const Gemm
     for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
     if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
 #else
-    epilogue_lds<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
 template <int BM, int BN, int WGM, int WGN, int EPI, int FEED>
 hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
-    constexpr int stage2 = 2 * (BM + BN) * ROW_BYTES, epi = epilogue_lds_bytes<BM, BN>();
+    constexpr int stage2 = 2 * (BM + BN) * ROW_BYTES, epi = epilogue_lds2_bytes<BM, BN>();
     constexpr int smem = stage2 > epi ? stage2 : epi;
     static bool configured = false;  // per instantiation; the attribute is idempotent
     auto kern = FEED == 3 ? gemm_nt_pipe4_kernel<BM, BN, WGM, WGN, EPI>
