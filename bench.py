@@ -185,7 +185,7 @@ def main():
     if "bx_axpy" in kernels:
         tot_ms, cnt = kern["bx_axpy"]
         achieved = bx_f * args.steps / (tot_ms * 1e-3) / 1e12
-        roofline = {"kernel": "gemm_nt_kernel<EPI_BX> (X' = a.X + B.X)", "bound": "mfma", "achieved": achieved,
+        roofline = {"kernel": "gemm_nt_*_kernel<256, 256, ..., EPI_BX> (X' = a.X + B.X)", "bound": "mfma", "achieved": achieved,
                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
                     "launches": cnt, "avg_launch_ms": tot_ms / cnt,
                     "algorithmic_flop_per_launch": bx_f * args.steps / cnt}

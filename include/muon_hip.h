@@ -63,6 +63,7 @@ extern "C" {
 /* 32-column k-tiles in four LDS stages: loads spread evenly between the MFMAs */
 #define MUON_HIP_CFG_128x128_W4_PIPE4 9
 #define MUON_HIP_CFG_256x256_W4_PIPE4 10
+#define MUON_HIP_CFG_256x256_W8_PIPE4 11
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);

@@ -978,6 +978,7 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
         case GEMM_CFG_256x256_W8_PIPE: return launch_one<256, 256, 2, 4, EPI, 2>(g, nblocks, stream);
         case GEMM_CFG_128x128_W4_PIPE4: return launch_one<128, 128, 2, 2, EPI, 3>(g, nblocks, stream);
         case GEMM_CFG_256x256_W4_PIPE4: return launch_one<256, 256, 2, 2, EPI, 3>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8_PIPE4: return launch_one<256, 256, 2, 4, EPI, 3>(g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -996,7 +997,8 @@ int gemm_cfg_tile(int cfg) {
         case GEMM_CFG_256x256_W8_DLDS:
         case GEMM_CFG_256x256_W4_PIPE:
         case GEMM_CFG_256x256_W8_PIPE:
-        case GEMM_CFG_256x256_W4_PIPE4: return 256;
+        case GEMM_CFG_256x256_W4_PIPE4:
+        case GEMM_CFG_256x256_W8_PIPE4: return 256;
         default: return 0;
     }
 }
