@@ -77,7 +77,7 @@ struct Plan {
     int ldx, ldxt, lda;  // row pitches (elements) of X, Xt and A/B
     bool transposed;
     long n, strideU, strideX, strideXT, strideA;
-    size_t offX[2], offXT[2], offA, offB, offParts, total;
+    size_t offX[2], offXT[2], offA, offB, offParts, offDenom, total;
 };
 
 constexpr int MUON_LD_PAD = 128;  // bf16 elements = 256 bytes
@@ -141,6 +141,7 @@ int make_plan(int rows, int cols, int batch, Plan& p) {
     p.offA = seg(ab);
     p.offB = seg(ab);
     p.offParts = seg((size_t)batch * p.nparts * sizeof(float));
+    p.offDenom = seg((size_t)batch * sizeof(float));
     p.total = off;
     return 0;
 }
@@ -315,8 +316,9 @@ int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int step
     bf16_t* B = wsp(workspace, p.offB);
     {
         Timed t(MUON_HIP_K_NORMALIZE, s);
-        hipError_t e = launch_normalize(X[1], p.strideU, (const float*)((char*)workspace + p.offParts), p.nparts, X[0],
-                                        p.ldx, p.strideX, XT[0], p.ldxt, p.strideXT, rows, cols, p.Mp, p.Kp, batch, s);
+        hipError_t e = launch_normalize(X[1], p.strideU, (const float*)((char*)workspace + p.offParts), p.nparts,
+                                        (float*)((char*)workspace + p.offDenom), X[0], p.ldx, p.strideX, XT[0], p.ldxt,
+                                        p.strideXT, rows, cols, p.Mp, p.Kp, batch, s);
         if (e != hipSuccess) return hip_fail(e, "normalize launch");
     }
     int cur = 0;

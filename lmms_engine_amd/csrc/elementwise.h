@@ -3,7 +3,7 @@
 #include <hip/hip_runtime.h>
 #include "common.h"
 
-#define MUON_MAX_PARTS 1024  // Frobenius partial sums per matrix, at most
+#define MUON_MAX_PARTS 4096  // Frobenius partial sums per matrix, at most
 
 int momentum_parts(long n);
 hipError_t launch_momentum_norm(const void* const* g_ptrs, const void* const* m_ptrs, int g_dtype, int m_dtype,
@@ -11,9 +11,9 @@ hipError_t launch_momentum_norm(const void* const* g_ptrs, const void* const* m_
                                 double beta, int nesterov, int write_back, hipStream_t stream);
 hipError_t launch_cast_norm(const void* G, long strideG, int g_dtype, bf16_t* U, long strideU, float* partials,
                             int nparts, long n, int batch, hipStream_t stream);
-hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, bf16_t* X, int ldx,
-                            long strideX, bf16_t* XT, int ldxt, long strideXT, int rows, int cols, int Mp, int Kp,
-                            int batch, hipStream_t stream);
+hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, float* denom, bf16_t* X,
+                            int ldx, long strideX, bf16_t* XT, int ldxt, long strideXT, int rows, int cols, int Mp,
+                            int Kp, int batch, hipStream_t stream);
 hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf16_t* O, long strideO, int ldo,
                                int rows, int cols, int batch, double scale, double lr, double wd,
                                hipStream_t stream);
