@@ -26,6 +26,11 @@ if ROOT not in sys.path:
 METRIC = "Muon step ms + NS TFLOP/s (% bf16 MFMA peak), Qwen3-8B param set, 1 GPU"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
+# Mean HBM-side bytes (L2 misses plus write-backs) of one B.X launch in a full step of each workload:
+# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over this script, each scaled by what the same counter
+# reads for the 1 GiB copy of --calibrate-copy (one FETCH_SIZE unit = 2 KiB, one WRITE_SIZE unit = 1 KiB).
+# A counter run cannot share a process with the event timing, so the figure is carried here.
+BX_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 18.516e9 + 5.001e9}
 
 WORKLOADS = {
     "qwen3-8b": dict(layers=36, shapes=dict(q=(4096, 4096), k=(1024, 4096), v=(1024, 4096), o=(4096, 4096),
@@ -108,6 +113,9 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the workload's own)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device copy (a kernel of known traffic) so that FETCH_SIZE / WRITE_SIZE "
+                         "readings of a rocprofv3 --pmc run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the Muon step on ONE GPU (no sharding, no collectives); use --gpus 1",
@@ -142,6 +150,12 @@ def main():
     flops_step = sum(ns_flops(*s, HP["ns_steps"]) for s in shapes)
     elements = sum(s[0] * s[1] for s in shapes)
 
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         opt.step()
     torch.cuda.synchronize()
@@ -186,7 +200,8 @@ def main():
         tot_ms, cnt = kern["bx_axpy"]
         achieved = bx_f * args.steps / (tot_ms * 1e-3) / 1e12
         roofline = {"kernel": "gemm_nt_*_kernel<256, 256, ..., EPI_BX> (X' = a.X + B.X)", "bound": "mfma", "achieved": achieved,
-                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                    "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
+                    "traffic": BX_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload) if layers == w["layers"] else None,
                     "launches": cnt, "avg_launch_ms": tot_ms / cnt,
                     "algorithmic_flop_per_launch": bx_f * args.steps / cnt}
     gemm_ms = sum(kernels[k]["ms_per_step"] for k in ("syrk", "sympoly", "bx_axpy") if k in kernels)

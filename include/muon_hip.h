@@ -64,6 +64,8 @@ extern "C" {
 #define MUON_HIP_CFG_128x128_W4_PIPE4 9
 #define MUON_HIP_CFG_256x256_W4_PIPE4 10
 #define MUON_HIP_CFG_256x256_W8_PIPE4 11
+/* two groups of four waves alternating between a memory phase and an MFMA-only phase */
+#define MUON_HIP_CFG_256x256_W8_PINGPONG 12
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);

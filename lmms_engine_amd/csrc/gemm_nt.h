@@ -17,7 +17,8 @@ enum {
     GEMM_CFG_128x128_W4_PIPE4 = 9,
     GEMM_CFG_256x256_W4_PIPE4 = 10,
     GEMM_CFG_256x256_W8_PIPE4 = 11,
-    GEMM_CFG_COUNT = 12
+    GEMM_CFG_256x256_W8_PINGPONG = 12,
+    GEMM_CFG_COUNT = 13
 };
 
 struct GemmArgs {

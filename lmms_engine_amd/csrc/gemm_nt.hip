@@ -14,6 +14,8 @@
 //
 // Operands are zero padded by the caller to whole tiles, so there is no masking here; the
 // host launcher checks that the shapes it is given are whole tiles before launching.
+#include <type_traits>
+
 #include "common.h"
 #include "gemm_nt.h"
 
@@ -63,6 +65,15 @@ __device__ __forceinline__ void rect_decode(int t, int TM, int TN, int& ti, int&
 struct TileCoord {
     int bidx, ti, tj;
 };
+
+// A pointer that is the same in every lane, moved into scalar registers.
+template <typename T>
+__device__ __forceinline__ const T* uniform_ptr(const T* p) {
+    const unsigned long long v = (unsigned long long)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return (const T*)(((unsigned long long)hi << 32) | lo);
+}
 
 // Every tile takes the same time, so without help all CUs reach their epilogues together and
 // the write-back arrives at HBM as one burst per round while the MFMAs idle.  Delaying the
@@ -716,7 +727,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     for (int n = 0; n < NRD; ++n) read_one(0, n, smem, 0);
 
 #ifdef EXP_TRACE
-    long long* trace = (long long*)g.Ct + (long)blockIdx.x * 4096 + (threadIdx.x >> 6) * 1024;
+    long long* trace = (long long*)g.Ct + (long)blockIdx.x * 8192 + (threadIdx.x >> 6) * 1024;
     int tn = 0;
 #define TRACE_POINT() do { if (lane == 0 && tn < 1000) trace[tn] = clock64(); ++tn; } while (0)
 #else
@@ -876,7 +887,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe4_kernel(const Gemm
     for (int n = 0; n < NRD; ++n) read_one(0, n, smem, 0);
 
 #ifdef EXP_TRACE
-    long long* trace = (long long*)g.Ct + (long)blockIdx.x * 4096 + (threadIdx.x >> 6) * 1024;
+    long long* trace = (long long*)g.Ct + (long)blockIdx.x * 8192 + (threadIdx.x >> 6) * 1024;
     int tn = 0;
 #endif
     for (int kt = 0; kt < nk; ++kt) {
@@ -946,12 +957,193 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe4_kernel(const Gemm
 #endif
 }
 
+// ---- variant 5: eight waves in two groups that alternate between memory and MFMA phases ----
+// Every wave runs the same loop  { M(t): read its fragments of k-tile t from LDS, issue its
+// share of the loads of k-tile t+3, wait;  barrier;  C(t): FM*FN*2 MFMAs;  barrier }  over
+// 32-column k-tiles in four LDS stages, but waves 4..7 enter it one barrier later than waves
+// 0..3.  Wave w and wave w+4 share a SIMD, so at any time one of them is issuing nothing but
+// MFMAs from registers while the other does all the LDS and address-path work and absorbs the
+// waits; the barrier is crossed when the MFMA wave has issued its last MFMA.
+// Timeline (phase p between two barriers): group 0 runs M(t) in p=2t and C(t) in p=2t+1,
+// group 1 runs M(t) in p=2t+1 and C(t) in p=2t+2.  Stage t&3 is last read in p=2t+1, the
+// loads of k-tile t+4 into it are issued in p=2t+2 / 2t+3, each wave waits for its own at the
+// end of its M phase two k-tiles later (p=2t+6 / 2t+7), and k-tile t+4 is first read in p=2t+8.
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArgs g) {
+    constexpr int NW = WGM * WGN;
+    constexpr int BK4 = 32, ROWB = 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int LA = BM / 16 / NW, LB = BN / 16 / NW;
+    constexpr int NLD = LA + LB;
+    static_assert(NW == 8, "two groups of four waves, one of each per SIMD");
+    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "dma split");
+    static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave >> 2;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const TileCoord tc = decode_tile<EPI>(g);
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+#ifdef EXPP_SAME_TILE
+    const bf16_t* Pb = uniform_ptr(g.P);
+    const bf16_t* Qb = uniform_ptr(g.Q);
+#else
+    const bf16_t* Pb = uniform_ptr(g.P + tc.bidx * g.strideP + m0 * g.ldp);
+    const bf16_t* Qb = uniform_ptr(g.Q + tc.bidx * g.strideQ + n0 * g.ldq);
+#endif
+
+    // Loads: a wave-uniform base pointer (advanced along k with scalar adds) plus a 32-bit byte
+    // offset per lane, so that no vector ALU instruction is needed per load: in the memory phase
+    // every VALU instruction would queue behind the sibling wave's MFMAs.
+    const int drow = lane >> 2;
+    const int dch = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;
+    unsigned offa[LA], offb[LB];
+#pragma unroll
+    for (int n = 0; n < LA; ++n) offa[n] = (unsigned)(((wave * 16 * LA + n * 16 + drow) * (long)g.ldp + dch) * 2);
+#pragma unroll
+    for (int n = 0; n < LB; ++n) offb[n] = (unsigned)(((wave * 16 * LB + n * 16 + drow) * (long)g.ldq + dch) * 2);
+    const int lds_a = wave * 16 * LA * ROWB;
+    const int lds_b = A_BYTES + wave * 16 * LB * ROWB;
+    const int nk = g.kdim / BK4;
+
+    // global_load_lds_dwordx4 with a scalar base and a 32-bit vector offset; the LDS destination
+    // of lane 0 goes through M0 (the wave's 64 lanes fill 1 KB from there in lane order).
+    auto dma = [&](const char* base, unsigned voff, unsigned lds_byte) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_byte), "v"(voff), "s"(base)
+                     : "memory");
+    };
+    const unsigned lds_base = (unsigned)(uintptr_t)(lds_void_ptr)smem;
+    auto issue_tile = [&](int kt) {  // kt may run past the end: re-load the last k-tile
+        const int kk = (kt < nk ? kt : nk - 1) * BK4;
+        const char* ba = (const char*)(Pb + kk);
+        const char* bb = (const char*)(Qb + kk);
+        const unsigned st = lds_base + (kt & 3) * STAGE;
+#pragma unroll
+        for (int n = 0; n < LA; ++n) dma(ba, offa[n], st + lds_a + n * 16 * ROWB);
+#pragma unroll
+        for (int n = 0; n < LB; ++n) dma(bb, offb[n], st + lds_b + n * 16 * ROWB);
+    };
+
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int sw = (lane >> 2) & 3, hi = lane >> 5;
+    const int a_off = (wm * WTM + (lane & 31)) * ROWB;
+    const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROWB;
+
+    issue_tile(0);
+    issue_tile(1);
+    issue_tile(2);
+    WAIT_VM(2 * NLD);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (grp) __builtin_amdgcn_s_barrier();
+
+#ifdef EXP_TRACE
+    long long* trace = (long long*)g.Ct + (long)blockIdx.x * 8192 + (threadIdx.x >> 6) * 1024;
+    int tn = 0;
+#endif
+    // LDS read addresses: one register per operand, k-step and pair of stages; the stage inside
+    // the pair and the fragment index are instruction offsets (below 64 KB) once the k loop is
+    // unrolled by the four stages.
+    const unsigned char* ra[2][2];
+    const unsigned char* rb[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const int co = (((ks << 1) | hi) ^ sw) << 4;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            ra[ks][half] = smem + half * 2 * STAGE + a_off + co;
+            rb[ks][half] = smem + half * 2 * STAGE + b_off + co;
+        }
+    }
+    auto body = [&](int kt, auto stage_c) {
+        constexpr int SIDX = decltype(stage_c)::value;
+        TRACE_POINT();
+        // ---- M(kt)
+        bf16x8 fa[2][FM], fb[2][FN];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+                fa[ks][i] = *(const bf16x8*)(ra[ks][SIDX >> 1] + (SIDX & 1) * STAGE + i * 32 * ROWB);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+                fb[ks][j] = *(const bf16x8*)(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 32 * ROWB);
+        }
+#ifndef EXPP_NO_DMA
+        issue_tile(kt + 3);
+#endif
+        TRACE_POINT();
+        WAIT_LGKM0();
+#ifndef EXPP_NO_DMA
+        WAIT_VM(2 * NLD);  // own loads of k-tile kt+1 have landed
+#endif
+        TRACE_POINT();
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        TRACE_POINT();
+        // ---- C(kt)
+#ifdef EXPP_SETPRIO
+        __builtin_amdgcn_s_setprio(3);
+#endif
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int i = 0; i < FM; ++i)
+#pragma unroll
+                for (int j = 0; j < FN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
+#ifdef EXPP_SETPRIO
+        __builtin_amdgcn_s_setprio(0);
+#endif
+        __builtin_amdgcn_sched_barrier(0);
+        TRACE_POINT();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // nk is a multiple of 4 (k extents are multiples of 128)
+    for (int kt = 0; kt < nk; kt += 4) {
+        body(kt, std::integral_constant<int, 0>{});
+        body(kt + 1, std::integral_constant<int, 1>{});
+        body(kt + 2, std::integral_constant<int, 2>{});
+        body(kt + 3, std::integral_constant<int, 3>{});
+    }
+    if (!grp) __builtin_amdgcn_s_barrier();
+    WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
+#ifdef EXP_NO_EPI
+    float ssum = 0.f;
+    for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
+    if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
+#else
+    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+#endif
+}
+
 template <int BM, int BN, int WGM, int WGN, int EPI, int FEED>
 hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
     constexpr int stage2 = 2 * (BM + BN) * ROW_BYTES, epi = epilogue_lds2_bytes<BM, BN>();
     constexpr int smem = stage2 > epi ? stage2 : epi;
     static bool configured = false;  // per instantiation; the attribute is idempotent
-    auto kern = FEED == 3 ? gemm_nt_pipe4_kernel<BM, BN, WGM, WGN, EPI>
+    auto kern = FEED == 4 ? gemm_nt_pp_kernel<BM, BN, 2, 4, EPI>
+              : FEED == 3 ? gemm_nt_pipe4_kernel<BM, BN, WGM, WGN, EPI>
               : FEED == 2 ? gemm_nt_pipe_kernel<BM, BN, WGM, WGN, EPI>
               : FEED == 1 ? gemm_nt_dlds_kernel<BM, BN, WGM, WGN, EPI>
                           : gemm_nt_kernel<BM, BN, WGM, WGN, EPI>;
@@ -979,6 +1171,7 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
         case GEMM_CFG_128x128_W4_PIPE4: return launch_one<128, 128, 2, 2, EPI, 3>(g, nblocks, stream);
         case GEMM_CFG_256x256_W4_PIPE4: return launch_one<256, 256, 2, 2, EPI, 3>(g, nblocks, stream);
         case GEMM_CFG_256x256_W8_PIPE4: return launch_one<256, 256, 2, 4, EPI, 3>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8_PINGPONG: return launch_one<256, 256, 2, 4, EPI, 4>(g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -998,7 +1191,8 @@ int gemm_cfg_tile(int cfg) {
         case GEMM_CFG_256x256_W4_PIPE:
         case GEMM_CFG_256x256_W8_PIPE:
         case GEMM_CFG_256x256_W4_PIPE4:
-        case GEMM_CFG_256x256_W8_PIPE4: return 256;
+        case GEMM_CFG_256x256_W8_PIPE4:
+        case GEMM_CFG_256x256_W8_PINGPONG: return 256;
         default: return 0;
     }
 }
