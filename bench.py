@@ -43,6 +43,9 @@ WORKLOADS = {
                               shapes=dict(q=(4096, 2048), k=(512, 2048), v=(512, 2048), o=(2048, 4096)),
                               expert_shapes=dict(gate=(768, 2048), up=(768, 2048), down=(2048, 768)),
                               pdtype="bf16", mdtype="f32"),
+    # single large matrices: the per-kernel MFMA utilisation sweep
+    "square-8192": dict(layers=1, shapes=dict(w=(8192, 8192)), pdtype="bf16", mdtype="f32"),
+    "llama70b-mlp-28672x8192": dict(layers=1, shapes=dict(w=(28672, 8192)), pdtype="bf16", mdtype="f32"),
 }
 HP = dict(lr=0.02, momentum=0.95, nesterov=True, weight_decay=0.01, ns_steps=5, rms_scale=False)
 

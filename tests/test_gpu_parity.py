@@ -458,6 +458,115 @@ def test_config2_full_size_sampled_parity(env):
         assert torch.isfinite(p).all()
 
 
+def _sv_band(out: torch.Tensor, probes: int = 8):
+    """Size-independent property of an orthogonalised matrix: five quintic iterations put every
+    singular value in about [0.55, 1.25], so ||out^T v|| / ||v|| (rows <= cols) stays in that band for
+    any v, and ||out||_F^2 / min(rows, cols) is the mean squared singular value.  fp64 on the CPU."""
+    o = out.double().cpu()
+    if o.shape[0] > o.shape[1]:
+        o = o.mT
+    gen = torch.Generator().manual_seed(5)
+    v = torch.randn(o.shape[0], probes, dtype=torch.float64, generator=gen)
+    ratio = (o.mT @ v).norm(dim=0) / v.norm(dim=0)
+    return ratio.min().item(), ratio.max().item(), (o.norm() ** 2 / o.shape[0]).item()
+
+
+@pytest.mark.parametrize("rows,cols", [(4096, 12288), (8192, 8192), (28672, 8192)])
+def test_full_size_newton_schulz(env, rows, cols):
+    """BASELINE config 3's largest shape and config 4's two matrices (N(0,1), seed 2, 5 iterations)
+    at full size: against the oracle on the host cores, and through properties that do not need it
+    (transpose equivariance and power-of-two scale invariance are exact; singular values land in the band)."""
+    print(f"full-size NS {rows}x{cols}", flush=True)
+    mu, O = env["mu"], env["O"]
+    G = torch.randn(rows, cols, generator=torch.Generator().manual_seed(2))
+    Gd = G.to(env["dev"])
+    out = mu.fast_newtonschulz(Gd, steps=5)
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16 and out.shape == (rows, cols) and torch.isfinite(out).all()
+    out_t = mu.fast_newtonschulz(Gd.mT.contiguous(), steps=5)
+    if rows != cols:
+        assert torch.equal(out_t, out.mT)  # the transpose rule makes both calls run the same arithmetic
+    else:
+        assert rel_fro(out_t, out.mT) <= NS_TOL  # a square matrix is iterated as given: equal only up to rounding
+    out_s = mu.fast_newtonschulz(Gd * 8.0, steps=5)
+    assert torch.equal(out_s, out)
+    lo, hi, mean_sq = _sv_band(out)
+    print(f"  sv probe band [{lo:.3f}, {hi:.3f}], mean s^2 {mean_sq:.3f}", flush=True)
+    assert 0.5 <= lo and hi <= 1.3 and 0.4 <= mean_sq <= 1.4
+    torch.set_num_threads(16)
+    ref = O.newton_schulz(G, 5)
+    err = rel_fro(out, ref)
+    print(f"  vs oracle {err:.3e}", flush=True)
+    assert err <= NS_TOL
+
+
+def test_config3_one_layer_full_step(env):
+    """BASELINE config 3 shapes (Qwen3-8B layer: bf16 params and grads, fp32 momentum), two layers so that
+    every bucket is a grouped launch; the oracle steps every matrix of layer 0 for two steps."""
+    print("config 3 layer", flush=True)
+    from tests.helpers import QWEN3_8B
+
+    mu, O, dev = env["mu"], env["O"], env["dev"]
+    weights, grads = make_param_set(QWEN3_8B, layers=2, seed=1, steps=2, dtype=torch.bfloat16)
+    gp = [torch.nn.Parameter(w.clone().to(dev)) for _, w in weights]
+    opt = mu.Muon([dict(params=list(gp), use_muon=True, **MUON_HP)], momentum_dtype=torch.float32)
+    sample = [i for i, (n, _) in enumerate(weights) if n.startswith("layers.0.")]
+    cw = {i: weights[i][1].clone() for i in sample}
+    cm = {i: torch.zeros(weights[i][1].shape, dtype=torch.float32) for i in sample}
+    torch.set_num_threads(16)
+    lr, wd = MUON_HP["lr"], MUON_HP["weight_decay"]
+    for step in range(2):
+        for p, g in zip(gp, grads[step]):
+            p.grad = g.to(dev)
+        opt.step()
+        torch.cuda.synchronize()
+        for i in sample:
+            O.muon_step_matrix(cw[i], grads[step][i].clone(), cm[i], lr=lr, weight_decay=wd, beta=MUON_HP["momentum"],
+                               nesterov=True, ns_steps=5, rms_scale=False)
+            assert rel_fro(opt.state[gp[i]]["momentum_buffer"], cm[i]) <= MOM_TOL, (step, weights[i][0])
+            # parameters are bf16: the two sides may round a few elements to neighbouring values
+            wp = rel_fro(gp[i], cw[i])
+            print(f"  step {step} {weights[i][0]}: param {wp:.3e}", flush=True)
+            assert wp <= 4e-3, (step, weights[i][0])
+
+
+def test_config5_moe_layer_sampled_parity(env):
+    """BASELINE config 5 shapes (Qwen3-MoE-30B-A3B: 128 experts x (gate, up 768x2048; down 2048x768) plus
+    attention q 4096x2048, k, v 512x2048, o 2048x4096; grads N(0, 1e-3) seed 3, bf16 params, fp32 momentum):
+    one full layer, 388 matrices in 5 grouped buckets; the oracle steps a sample out of every bucket."""
+    print("config 5 layer", flush=True)
+    mu, O, dev = env["mu"], env["O"], env["dev"]
+    gen = torch.Generator().manual_seed(3)
+    shapes = [("q", (4096, 2048)), ("k", (512, 2048)), ("v", (512, 2048)), ("o", (2048, 4096))]
+    for e in range(128):
+        shapes += [(f"e{e}.gate", (768, 2048)), (f"e{e}.up", (768, 2048)), (f"e{e}.down", (2048, 768))]
+    weights = [(n, (0.02 * torch.randn(*s, generator=gen)).bfloat16()) for n, s in shapes]
+    grads = [(1e-3 * torch.randn(*s, generator=gen)).bfloat16() for _, s in shapes]
+    gp = [torch.nn.Parameter(w.clone().to(dev)) for _, w in weights]
+    for p, g in zip(gp, grads):
+        p.grad = g.to(dev)
+    opt = mu.Muon([dict(params=list(gp), use_muon=True, **MUON_HP)], momentum_dtype=torch.float32)
+    before = [p.detach().clone() for p in gp]
+    opt.step()
+    torch.cuda.synchronize()
+    lr, wd = MUON_HP["lr"], MUON_HP["weight_decay"]
+    names = [n for n, _ in weights]
+    sample = [names.index(n) for n in ("q", "k", "o", "e0.gate", "e0.down", "e77.up", "e127.gate", "e127.down")]
+    for i in sample:
+        w, m = weights[i][1].clone(), torch.zeros(weights[i][1].shape, dtype=torch.float32)
+        O.muon_step_matrix(w, grads[i].clone(), m, lr=lr, weight_decay=wd, beta=MUON_HP["momentum"], nesterov=True,
+                           ns_steps=5, rms_scale=False)
+        assert rel_fro(opt.state[gp[i]]["momentum_buffer"], m) <= MOM_TOL, names[i]
+        assert rel_fro(gp[i], w) <= 4e-3, names[i]
+    # every matrix moved by an update whose size matches an orthogonalised one:
+    # ||dp||_F ~ lr * sqrt(min(rows, cols)) * sqrt(max(1, rows / cols)), up to the bf16 rounding of p
+    for i, p in enumerate(gp):
+        assert torch.isfinite(p).all()
+        d = (p.detach().float() - before[i].float() * (1 - lr * wd)).norm().item() / lr
+        r = d / (min(p.shape) ** 0.5) / max(1.0, p.shape[0] / p.shape[1]) ** 0.5
+        assert 0.5 <= r <= 1.3, (names[i], r)
+
+
 def test_golden_vectors_on_gpu(env):
     """The committed golden vectors (tests/golden/, written by make_fixtures.py from the oracle)."""
     import os
