@@ -66,6 +66,8 @@ extern "C" {
 #define MUON_HIP_CFG_256x256_W8_PIPE4 11
 /* two groups of four waves alternating between a memory phase and an MFMA-only phase */
 #define MUON_HIP_CFG_256x256_W8_PINGPONG 12
+/* the same with five LDS stages (all 160 KB): loads stay in flight one k-tile longer */
+#define MUON_HIP_CFG_256x256_W8_PINGPONG5 13
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);

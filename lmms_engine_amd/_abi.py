@@ -19,8 +19,8 @@ CFG_AUTO, CFG_128x128_W4, CFG_256x256_W4, CFG_256x256_W8 = -1, 0, 1, 2
 CFG_128x128_W4_DLDS, CFG_256x256_W4_DLDS, CFG_256x256_W8_DLDS = 3, 4, 5
 CFG_128x128_W4_PIPE, CFG_256x256_W4_PIPE, CFG_256x256_W8_PIPE = 6, 7, 8
 CFG_128x128_W4_PIPE4, CFG_256x256_W4_PIPE4, CFG_256x256_W8_PIPE4 = 9, 10, 11
-CFG_256x256_W8_PINGPONG = 12
-GEMM_CONFIGS = list(range(13))
+CFG_256x256_W8_PINGPONG, CFG_256x256_W8_PINGPONG5 = 12, 13
+GEMM_CONFIGS = list(range(14))
 K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW = range(7)
 KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw"]
 

@@ -18,7 +18,8 @@ enum {
     GEMM_CFG_256x256_W4_PIPE4 = 10,
     GEMM_CFG_256x256_W8_PIPE4 = 11,
     GEMM_CFG_256x256_W8_PINGPONG = 12,
-    GEMM_CFG_COUNT = 13
+    GEMM_CFG_256x256_W8_PINGPONG5 = 13,
+    GEMM_CFG_COUNT = 14
 };
 
 struct GemmArgs {

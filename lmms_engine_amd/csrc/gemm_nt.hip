@@ -386,6 +386,145 @@ __device__ __forceinline__ void epilogue_lds2(const GemmArgs& g, const TileCoord
     }
 }
 
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// Epilogue with one LDS copy of the tile and both output orientations written as 16-byte
+// vectors.  The tile lives in LDS as Tt[n][m] (n = local column, m = local row of the
+// accumulator tile), the orientation of Ct and of the elementwise source Et: Et is loaded
+// into it with coalesced reads, every lane replaces its own 8-byte pieces (4 consecutive m of
+// one n, exactly what an accumulator lane holds) by the rounded results, and after one barrier
+// rows of Tt leave as rows of Ct, while rows of C are gathered with ds_read_b64_tr_b16: in a
+// group of 16 lanes, lane i receives element i%4 of the 8-byte pieces addressed by lanes
+// i/4, 4+i/4, 8+i/4, 12+i/4, so pointing lane j at row n0+j/4, pieces m0+4*(j%4).. hands lane
+// i the four values Tt[n0..n0+3][m0+i], i.e. 8 bytes of row m0+i of C.
+#ifndef EPI3_PITCH_PAD
+#define EPI3_PITCH_PAD 16
+#endif
+template <int BM, int BN>
+constexpr int epilogue_lds3_bytes() { return BN * (BM * 2 + EPI3_PITCH_PAD); }
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ s16x4 lds_read_tr16(const unsigned char* p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(lds_void_ptr)p);
+}
+
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__device__ __forceinline__ void epilogue_lds3(const GemmArgs& g, const TileCoord& tc,
+                                              f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], unsigned char* smem) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int S = BM * 2 + EPI3_PITCH_PAD;  // Tt row pitch (bytes)
+    constexpr int CPR = BM / 8;                 // 16-byte chunks per Tt row
+    constexpr int NLE = BN * CPR / NT;          // 16-byte chunks per thread for a whole tile
+    static_assert((BN * CPR) % NT == 0, "even split");
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN, hi = lane >> 5;
+    const long m0 = (long)tc.ti * BM, n0 = (long)tc.tj * BN;
+    const bool diag = (EPI != EPI_BX) && (tc.ti == tc.tj);
+    bf16_t* C = (g.C && !diag) ? g.C + tc.bidx * g.strideC + m0 * g.ldc + n0 : nullptr;
+    bf16_t* Ct = g.Ct ? g.Ct + tc.bidx * g.strideCt + n0 * g.ldct + m0 : nullptr;
+    EPI_POINT(0);
+    __syncthreads();  // the operand stages are no longer read
+    EPI_POINT(1);
+    if (EPI != EPI_SYRK) {
+        const bf16_t* Et = g.Et + tc.bidx * g.strideEt + n0 * g.ldet + m0;
+#pragma unroll
+        for (int b = 0; b < NLE; b += 16) {
+            u32x4 ev[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int c = tid + (b + u) * NT, n = c / CPR, k = c % CPR;
+                if (b + u < NLE) ev[u] = *(const u32x4*)(Et + (long)n * g.ldet + k * 8);
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int c = tid + (b + u) * NT, n = c / CPR, k = c % CPR;
+                if (b + u < NLE) *(u32x4*)(smem + n * S + k * 16) = ev[u];
+            }
+        }
+        __syncthreads();
+    }
+    EPI_POINT(2);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        // all LDS reads of a fragment row first: in one loop the compiler must assume that each
+        // write may alias the next read and the chain becomes one LDS latency per item
+        bf16x4 e[FN][4];
+        if (EPI != EPI_SYRK) {
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    e[j][q] = *(const bf16x4*)(smem + (wn * WTN + j * 32 + (lane & 31)) * S +
+                                               (wm * WTM + i * 32 + q * 8 + hi * 4) * 2);
+        }
+        bf16x4 o[FN][4];
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float v = rbf(acc[i][j][q * 4 + r]);
+                    if (EPI == EPI_SYMPOLY) v = rbf(rbf(g.s0 * bf2f(e[j][q][r])) + rbf(g.s1 * v));
+                    if (EPI == EPI_BX) v = rbf(rbf(g.s0 * bf2f(e[j][q][r])) + v);
+                    o[j][q][r] = f2bf(v);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                *(bf16x4*)(smem + (wn * WTN + j * 32 + (lane & 31)) * S + (wm * WTM + i * 32 + q * 8 + hi * 4) * 2) =
+                    o[j][q];
+    }
+    EPI_POINT(3);
+    __syncthreads();
+    EPI_POINT(4);
+    if (Ct) {
+#pragma unroll
+        for (int u = 0; u < NLE; ++u) {
+            const int c = tid + u * NT, n = c / CPR, k = c % CPR;
+            *(u32x4*)(Ct + (long)n * g.ldct + k * 8) = *(const u32x4*)(smem + n * S + k * 16);
+        }
+    }
+    EPI_POINT(5);
+    if (C) {
+        // lane j = 4r+s of a group addresses row n0 + 8s + r (then + 4), pieces m = 4c..4c+3: lane i = 4s+e
+        // receives Tt[n0+8s .. n0+8s+7][4c+e], 16 bytes of row 4c+e of C.  A group writes 4 rows x 64
+        // contiguous bytes and the four groups of a wave sit side by side: 4 rows x 256 bytes per store.
+        const int grp = lane >> 4, i16 = lane & 15;
+        const unsigned char* src = smem + ((i16 & 3) * 8 + (i16 >> 2) + grp * 32) * S;
+        bf16_t* dst = C + (long)(i16 & 3) * g.ldc + grp * 32 + (i16 >> 2) * 8;
+        constexpr int NSTRIP = BN / 128, NQUAD = BM / 4, NW = NT / 64;
+        constexpr int NUNIT = NSTRIP * NQUAD / NW;
+        static_assert(BN % 128 == 0 && (NSTRIP * NQUAD) % NW == 0, "whole 128-column strips per wave");
+#pragma unroll 8
+        for (int u = 0; u < NUNIT; ++u) {
+            const int wu = wave + u * NW, strip = wu % NSTRIP, c = wu / NSTRIP;
+            const unsigned char* q = src + strip * 128 * S + c * 8;
+            const s16x4 lo = lds_read_tr16(q), hi4 = lds_read_tr16(q + 4 * S);
+            short __attribute__((ext_vector_type(8))) o = {lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+            *(decltype(o)*)(dst + (long)c * 4 * g.ldc + strip * 128) = o;
+        }
+    }
+    EPI_POINT(6);
+#ifdef EXP_TRACE_EPI
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    EPI_POINT(7);
+#endif
+}
+
+#ifdef EXP_EPI_LDS2
+#define EPILOGUE epilogue_lds2
+#define EPILOGUE_BYTES epilogue_lds2_bytes
+#else
+#define EPILOGUE epilogue_lds3
+#define EPILOGUE_BYTES epilogue_lds3_bytes
+#endif
+
 // ---- variant 1: global -> registers -> LDS, two LDS stages, one barrier per k-tile -------
 template <int BM, int BN, int WGM, int WGN, int EPI>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g) {
@@ -474,7 +613,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g
 #elif defined(EXP_DIRECT_EPI)
     epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc);
 #else
-    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    EPILOGUE<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
@@ -483,7 +622,6 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_kernel(const GemmArgs g
 // the XOR swizzle is applied on the global side: lane L fetches the chunk whose swizzled
 // position is L&7.  Loads for k-tile t+2 are issued as soon as every wave has finished
 // reading k-tile t, and are waited for (vmcnt) one whole tile of MFMA work later.
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
 typedef const __attribute__((address_space(1))) void* glb_void_ptr;
 
 #define WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
@@ -621,7 +759,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_dlds_kernel(const GemmA
 #elif defined(EXP_DIRECT_EPI)
     epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc);
 #else
-    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    EPILOGUE<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
@@ -784,7 +922,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
     if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
 #else
-    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    EPILOGUE<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
@@ -953,7 +1091,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe4_kernel(const Gemm
     for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
     if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
 #else
-    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    EPILOGUE<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
@@ -968,7 +1106,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe4_kernel(const Gemm
 // group 1 runs M(t) in p=2t+1 and C(t) in p=2t+2.  Stage t&3 is last read in p=2t+1, the
 // loads of k-tile t+4 into it are issued in p=2t+2 / 2t+3, each wave waits for its own at the
 // end of its M phase two k-tiles later (p=2t+6 / 2t+7), and k-tile t+4 is first read in p=2t+8.
-template <int BM, int BN, int WGM, int WGN, int EPI>
+template <int BM, int BN, int WGM, int WGN, int EPI, int NST>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArgs g) {
     constexpr int NW = WGM * WGN;
     constexpr int BK4 = 32, ROWB = 64;
@@ -978,6 +1116,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
     constexpr int LA = BM / 16 / NW, LB = BN / 16 / NW;
     constexpr int NLD = LA + LB;
     static_assert(NW == 8, "two groups of four waves, one of each per SIMD");
+    static_assert(NST == 4 || NST == 5, "four or five LDS stages");
     static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "dma split");
     static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
 
@@ -1013,22 +1152,49 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
 
     // global_load_lds_dwordx4 with a scalar base and a 32-bit vector offset; the LDS destination
     // of lane 0 goes through M0 (the wave's 64 lanes fill 1 KB from there in lane order).
+#ifdef EXPP_TO_VGPR
+    f32x4 sink[4] = {};
+    int sink_i = 0;
     auto dma = [&](const char* base, unsigned voff, unsigned lds_byte) {
+        asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(sink[0]) : "v"(voff), "s"(base) : "memory");
+    };
+#else
+#ifdef EXPP_DWORD
+    auto dma = [&](const char* base, unsigned voff, unsigned lds_byte) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                     :
+                     : "s"(lds_byte), "v"(voff), "s"(base)
+                     : "memory");
+    };
+#else
+    auto dma = [&](const char* base, unsigned voff, unsigned lds_byte) {
+#ifdef EXPP_L1_HIT
+        voff = lane * 16; base = (const char*)Pb;
+#endif
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
                      : "s"(lds_byte), "v"(voff), "s"(base)
                      : "memory");
     };
+#endif
+#endif
     const unsigned lds_base = (unsigned)(uintptr_t)(lds_void_ptr)smem;
-    auto issue_tile = [&](int kt) {  // kt may run past the end: re-load the last k-tile
+    // load n (0..NLD-1) of k-tile kt into LDS stage `stage`; kt may run past the end: re-load the last k-tile
+    auto issue_one = [&](int kt, int stage, int n) {
+#ifdef EXPP_KWRAP
+        const int kk = ((kt < nk ? kt : nk - 1) & (EXPP_KWRAP - 1)) * BK4;
+#else
         const int kk = (kt < nk ? kt : nk - 1) * BK4;
-        const char* ba = (const char*)(Pb + kk);
-        const char* bb = (const char*)(Qb + kk);
-        const unsigned st = lds_base + (kt & 3) * STAGE;
+#endif
+        const unsigned st = lds_base + stage * STAGE;
+        if (n < LA)
+            dma((const char*)(Pb + kk), offa[n], st + lds_a + n * 16 * ROWB);
+        else
+            dma((const char*)(Qb + kk), offb[n - LA], st + lds_b + (n - LA) * 16 * ROWB);
+    };
+    auto issue_tile = [&](int kt, int stage) {
 #pragma unroll
-        for (int n = 0; n < LA; ++n) dma(ba, offa[n], st + lds_a + n * 16 * ROWB);
-#pragma unroll
-        for (int n = 0; n < LB; ++n) dma(bb, offb[n], st + lds_b + n * 16 * ROWB);
+        for (int n = 0; n < NLD; ++n) issue_one(kt, stage, n);
     };
 
     f32x16 acc[FM][FN];
@@ -1043,10 +1209,9 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
     const int a_off = (wm * WTM + (lane & 31)) * ROWB;
     const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROWB;
 
-    issue_tile(0);
-    issue_tile(1);
-    issue_tile(2);
-    WAIT_VM(2 * NLD);
+#pragma unroll
+    for (int t = 0; t < NST - 1; ++t) issue_tile(t, t);
+    WAIT_VM((NST - 2) * NLD);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     if (grp) __builtin_amdgcn_s_barrier();
@@ -1058,39 +1223,49 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
     // LDS read addresses: one register per operand, k-step and pair of stages; the stage inside
     // the pair and the fragment index are instruction offsets (below 64 KB) once the k loop is
     // unrolled by the four stages.
-    const unsigned char* ra[2][2];
-    const unsigned char* rb[2][2];
+    constexpr int NPAIR = (NST + 1) / 2;
+    const unsigned char* ra[2][NPAIR];
+    const unsigned char* rb[2][NPAIR];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
         const int co = (((ks << 1) | hi) ^ sw) << 4;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
+        for (int half = 0; half < NPAIR; ++half) {
             ra[ks][half] = smem + half * 2 * STAGE + a_off + co;
             rb[ks][half] = smem + half * 2 * STAGE + b_off + co;
         }
     }
-    auto body = [&](int kt, auto stage_c) {
+    auto body = [&](int kt, auto stage_c, auto masked_c) {
         constexpr int SIDX = decltype(stage_c)::value;
+        constexpr bool MASKED = decltype(masked_c)::value;
         TRACE_POINT();
         // ---- M(kt)
+        // The loads are throttled by the 64 B/clk path into the CU and the reads by LDS bandwidth:
+        // interleaved, the two queues drain side by side instead of one after the other.
         bf16x8 fa[2][FM], fb[2][FN];
+        constexpr int NRD = 2 * (FM + FN), RD_PER_LD = (NRD + NLD - 1) / NLD;
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-            for (int i = 0; i < FM; ++i)
-                fa[ks][i] = *(const bf16x8*)(ra[ks][SIDX >> 1] + (SIDX & 1) * STAGE + i * 32 * ROWB);
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-                fb[ks][j] = *(const bf16x8*)(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 32 * ROWB);
-        }
+        for (int r = 0; r < NRD; ++r) {
 #ifndef EXPP_NO_DMA
-        issue_tile(kt + 3);
+            if (r % RD_PER_LD == 0 && r / RD_PER_LD < NLD) issue_one(kt + NST - 1, (SIDX + NST - 1) % NST, r / RD_PER_LD);
 #endif
+            const int ks = r / (FM + FN), o = r % (FM + FN);
+            if (o < FM)
+                fa[ks][o] = *(const bf16x8*)(ra[ks][SIDX >> 1] + (SIDX & 1) * STAGE + o * 32 * ROWB);
+            else
+                fb[ks][o - FM] = *(const bf16x8*)(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + (o - FM) * 32 * ROWB);
+        }
         TRACE_POINT();
         WAIT_LGKM0();
 #ifndef EXPP_NO_DMA
-        WAIT_VM(2 * NLD);  // own loads of k-tile kt+1 have landed
+        WAIT_VM((NST - 2) * NLD);  // own loads of k-tile kt+1 have landed
 #endif
+        if (MASKED && kt >= nk) {  // a k-tile past the end (only in the peeled last group) contributes nothing
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int i = 0; i < FM; ++i) fa[ks][i] = bf16x8{};
+        }
         TRACE_POINT();
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" ::: "memory");
@@ -1119,30 +1294,50 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
         asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
     };
-    // nk is a multiple of 4 (k extents are multiples of 128)
-    for (int kt = 0; kt < nk; kt += 4) {
-        body(kt, std::integral_constant<int, 0>{});
-        body(kt + 1, std::integral_constant<int, 1>{});
-        body(kt + 2, std::integral_constant<int, 2>{});
-        body(kt + 3, std::integral_constant<int, 3>{});
+    using std::integral_constant;
+    if constexpr (NST == 4) {  // nk is a multiple of 4 (k extents are multiples of 128)
+        for (int kt = 0; kt < nk; kt += 4) {
+            body(kt, integral_constant<int, 0>{}, integral_constant<bool, false>{});
+            body(kt + 1, integral_constant<int, 1>{}, integral_constant<bool, false>{});
+            body(kt + 2, integral_constant<int, 2>{}, integral_constant<bool, false>{});
+            body(kt + 3, integral_constant<int, 3>{}, integral_constant<bool, false>{});
+        }
+    } else {  // groups of five k-tiles; the last group is peeled and masks the k-tiles past the end
+        int kt = 0;
+        for (; kt + 5 < nk; kt += 5) {
+            body(kt, integral_constant<int, 0>{}, integral_constant<bool, false>{});
+            body(kt + 1, integral_constant<int, 1>{}, integral_constant<bool, false>{});
+            body(kt + 2, integral_constant<int, 2>{}, integral_constant<bool, false>{});
+            body(kt + 3, integral_constant<int, 3>{}, integral_constant<bool, false>{});
+            body(kt + 4, integral_constant<int, 4>{}, integral_constant<bool, false>{});
+        }
+        body(kt, integral_constant<int, 0>{}, integral_constant<bool, true>{});
+        body(kt + 1, integral_constant<int, 1>{}, integral_constant<bool, true>{});
+        body(kt + 2, integral_constant<int, 2>{}, integral_constant<bool, true>{});
+        body(kt + 3, integral_constant<int, 3>{}, integral_constant<bool, true>{});
+        body(kt + 4, integral_constant<int, 4>{}, integral_constant<bool, true>{});
     }
     if (!grp) __builtin_amdgcn_s_barrier();
     WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
 #ifdef EXP_NO_EPI
     float ssum = 0.f;
     for (int i = 0; i < FM; ++i) for (int j = 0; j < FN; ++j) for (int r = 0; r < 16; ++r) ssum += acc[i][j][r];
+#ifdef EXPP_TO_VGPR
+    ssum += sink[0][0] + sink[0][1] + sink[0][2] + sink[0][3];
+#endif
     if (ssum == 123.456f) g.C[threadIdx.x] = f2bf(ssum);
 #else
-    epilogue_lds2<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    EPILOGUE<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 #endif
 }
 
 template <int BM, int BN, int WGM, int WGN, int EPI, int FEED>
 hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
-    constexpr int stage2 = 2 * (BM + BN) * ROW_BYTES, epi = epilogue_lds2_bytes<BM, BN>();
+    constexpr int stage2 = FEED == 5 ? 5 * (BM + BN) * 64 : 2 * (BM + BN) * ROW_BYTES, epi = EPILOGUE_BYTES<BM, BN>();
     constexpr int smem = stage2 > epi ? stage2 : epi;
     static bool configured = false;  // per instantiation; the attribute is idempotent
-    auto kern = FEED == 4 ? gemm_nt_pp_kernel<BM, BN, 2, 4, EPI>
+    auto kern = FEED == 5 ? gemm_nt_pp_kernel<BM, BN, 2, 4, EPI, 5>
+              : FEED == 4 ? gemm_nt_pp_kernel<BM, BN, 2, 4, EPI, 4>
               : FEED == 3 ? gemm_nt_pipe4_kernel<BM, BN, WGM, WGN, EPI>
               : FEED == 2 ? gemm_nt_pipe_kernel<BM, BN, WGM, WGN, EPI>
               : FEED == 1 ? gemm_nt_dlds_kernel<BM, BN, WGM, WGN, EPI>
@@ -1172,6 +1367,7 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
         case GEMM_CFG_256x256_W4_PIPE4: return launch_one<256, 256, 2, 2, EPI, 3>(g, nblocks, stream);
         case GEMM_CFG_256x256_W8_PIPE4: return launch_one<256, 256, 2, 4, EPI, 3>(g, nblocks, stream);
         case GEMM_CFG_256x256_W8_PINGPONG: return launch_one<256, 256, 2, 4, EPI, 4>(g, nblocks, stream);
+        case GEMM_CFG_256x256_W8_PINGPONG5: return launch_one<256, 256, 2, 4, EPI, 5>(g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -1192,7 +1388,8 @@ int gemm_cfg_tile(int cfg) {
         case GEMM_CFG_256x256_W8_PIPE:
         case GEMM_CFG_256x256_W4_PIPE4:
         case GEMM_CFG_256x256_W8_PIPE4:
-        case GEMM_CFG_256x256_W8_PINGPONG: return 256;
+        case GEMM_CFG_256x256_W8_PINGPONG:
+        case GEMM_CFG_256x256_W8_PINGPONG5: return 256;
         default: return 0;
     }
 }
