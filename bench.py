@@ -107,6 +107,43 @@ def cpu_baseline(w, layers, target_flops_per_step):
     }
 
 
+def extras(params, pd, dev, reps):
+    """Gradient clipping over the Muon gradients and the AdamW fallback over a Qwen3-8B-shaped non-Muon group
+    (embedding and lm_head 151936x4096, 73 norm vectors), each as achieved HBM bytes per second."""
+    import torch
+
+    from lmms_engine_amd import _abi
+    from lmms_engine_amd.clip_grad import clip_grad_norm_
+    from lmms_engine_amd.muon_utils import Muon
+
+    gb = 2 if pd == torch.bfloat16 else 4
+    shapes = [(151936, 4096), (151936, 4096)] + [(4096,)] * 73
+    fb = [torch.nn.Parameter(torch.zeros(*s, dtype=pd, device=dev)) for s in shapes]
+    for p in fb:
+        p.grad = torch.full_like(p, 1e-3)
+    opt = Muon([dict(params=fb, use_muon=False, lr=1e-4, betas=(0.9, 0.95), eps=1e-8, weight_decay=0.01)])
+    opt.step()
+    clip_grad_norm_(params, 1.0)
+    torch.cuda.synchronize()
+    _abi.timing_enable(True)
+    for _ in range(reps):
+        clip_grad_norm_(params, 1.0)
+        opt.step()
+    torch.cuda.synchronize()
+    t = _abi.timing_read()
+    _abi.timing_enable(False)
+    n_muon = sum(p.numel() for p in params)
+    n_fb = sum(p.numel() for p in fb)
+    res = {}
+    for name, nbytes in (("grad_norm", n_muon * gb), ("clip_scale", n_muon * 2 * gb), ("adamw_multi", n_fb * 7 * gb)):
+        ms, cnt = t[name]
+        if cnt:
+            per = ms / reps
+            res[name] = dict(ms_per_call=per, launches_per_call=cnt / reps, gbs=nbytes / (per * 1e-3) / 1e9,
+                             frac_hbm_peak=nbytes / (per * 1e-3) / 1e9 / PEAK_HBM_GBS)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -116,6 +153,9 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the workload's own)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--extras", action="store_true",
+                    help="also time the two neighbours of the Muon step, outside the timed region: gradient-norm clipping "
+                         "over the same gradients and the AdamW fallback over an embedding + lm_head + norm-vector group")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic) so that FETCH_SIZE / WRITE_SIZE "
                          "readings of a rocprofv3 --pmc run can be scaled")
@@ -231,6 +271,8 @@ def main():
         "kernels": kernels,
         "roofline": roofline,
     }
+    if args.extras:
+        out["extras"] = extras(params, pd, dev, args.steps)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, layers, flops_step)
     print(json.dumps(out))

@@ -45,7 +45,10 @@ extern "C" {
 #define MUON_HIP_K_BX 4
 #define MUON_HIP_K_UPDATE 5
 #define MUON_HIP_K_ADAMW 6
-#define MUON_HIP_K_COUNT 7
+#define MUON_HIP_K_ADAMW_MULTI 7
+#define MUON_HIP_K_GRAD_NORM 8
+#define MUON_HIP_K_CLIP_SCALE 9
+#define MUON_HIP_K_COUNT 10
 
 /* GEMM tile configurations; MUON_HIP_CFG_AUTO picks by shape. */
 #define MUON_HIP_CFG_AUTO (-1)
@@ -151,6 +154,40 @@ int muon_hip_bx_axpy_bf16(const void* B, int lda, const void* XT, int ldxt, void
  * tensor of n elements; p, g, exp_avg, exp_avg_sq share `dtype`; `step` is already incremented. */
 int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int dtype, long n, int step, double lr,
                    double beta1, double beta2, double eps, double weight_decay, void* stream);
+
+/* ---- multi-tensor kernels ---------------------------------------------------------------
+ * One launch walks a list of n tensors of one dtype.  The list is described by device arrays:
+ * base pointers (`const void* const*`, n entries), element counts `numel` (n longs) and
+ * `chunk_start` (n + 1 longs): tensors are cut into chunks of MUON_HIP_MULTI_CHUNK elements,
+ * chunk_start[t] is the index of tensor t's first chunk and chunk_start[n] == chunks, the total
+ * (one workgroup per chunk).  The caller builds these arrays; the library cannot check them. */
+#define MUON_HIP_MULTI_CHUNK 16384
+
+/* The Adam branch of step_fsdp over a whole parameter group in one launch: adam_update
+ * (muon_utils.py:178-183) then decay and update (:473-477), i.e. muon_hip_adamw for every tensor
+ * of the list.  bias1[t] = 1 - beta1**step_t and bias2[t] = 1 - beta2**step_t (device doubles,
+ * steps already incremented: each parameter keeps its own step, muon_utils.py:471). */
+int muon_hip_adamw_multi(const void* const* p_ptrs, const void* const* g_ptrs, const void* const* exp_avg_ptrs,
+                         const void* const* exp_avg_sq_ptrs, const long* numel, const long* chunk_start,
+                         const double* bias1, const double* bias2, int n, long chunks, int dtype, double lr,
+                         double beta1, double beta2, double eps, double weight_decay, void* stream);
+
+/* Gradient clipping, the step before optimizer.step(): fsdp2_clip_grad_norm_ on one device
+ * (utils/fsdp2_utils.py:234-255) is torch's _get_total_norm + _clip_grads_with_norm_ with the
+ * 2-norm.
+ * muon_hip_grad_norms: norms[t] = ||g_t||_2 accumulated in fp32 and rounded to the tensors' dtype,
+ *   as fp32 values (the per-tensor norms of torch._foreach_norm); `partials` is scratch of
+ *   `chunks` floats.
+ * muon_hip_total_norm: the norm of n such norms (lists of several dtypes concatenated by the
+ *   caller), rounded to `dtype`, written as fp32 to *total_f32 and in `dtype` to *total_typed.
+ * muon_hip_clip_scale: g_t *= min(1, max_norm / (total + 1e-6)) for every tensor of the list,
+ *   the coefficient evaluated as torch does, (total + 1e-6).reciprocal() * max_norm in the
+ *   norm's dtype `norm_dtype`, read from device memory so that no host synchronisation is needed. */
+int muon_hip_grad_norms(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
+                        int dtype, float* partials, float* norms, void* stream);
+int muon_hip_total_norm(const float* norms, int n, int dtype, float* total_f32, void* total_typed, void* stream);
+int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
+                        int dtype, const float* total_f32, int norm_dtype, double max_norm, void* stream);
 
 /* ---- per-kernel timing ----------------------------------------------------------------
  * No counterpart in the reference.  When enabled, every kernel launch is bracketed by a pair

@@ -21,8 +21,10 @@ CFG_128x128_W4_PIPE, CFG_256x256_W4_PIPE, CFG_256x256_W8_PIPE = 6, 7, 8
 CFG_128x128_W4_PIPE4, CFG_256x256_W4_PIPE4, CFG_256x256_W8_PIPE4 = 9, 10, 11
 CFG_256x256_W8_PINGPONG, CFG_256x256_W8_PINGPONG5 = 12, 13
 GEMM_CONFIGS = list(range(14))
-K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW = range(7)
-KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw"]
+K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW, K_ADAMW_MULTI, K_GRAD_NORM, K_CLIP_SCALE = range(10)
+KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw", "adamw_multi",
+                "grad_norm", "clip_scale"]
+MULTI_CHUNK = 16384  # MUON_HIP_MULTI_CHUNK
 
 # name -> (restype, argtypes); mirrors include/muon_hip.h one to one
 SIGNATURES = {
@@ -47,6 +49,11 @@ SIGNATURES = {
                                       c_double, c_int, c_void_p]),
     "muon_hip_adamw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_double,
                                c_double, c_double, c_double, c_void_p]),
+    "muon_hip_adamw_multi": (c_int, [c_void_p] * 8 + [c_int, c_long, c_int] + [c_double] * 5 + [c_void_p]),
+    "muon_hip_grad_norms": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_void_p, c_void_p]),
+    "muon_hip_total_norm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "muon_hip_clip_scale": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_int, c_double,
+                                    c_void_p]),
     "muon_hip_timing_enable": (c_int, [c_int]),
     "muon_hip_timing_read": (c_int, [c_int, POINTER(c_double), POINTER(c_long)]),
 }

@@ -9,6 +9,7 @@
 #include "common.h"
 #include "elementwise.h"
 #include "gemm_nt.h"
+#include "multi_tensor.h"
 
 namespace {
 
@@ -420,6 +421,59 @@ int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int 
     Timed t(MUON_HIP_K_ADAMW, s);
     hipError_t e = launch_adamw(p, g, exp_avg, exp_avg_sq, dtype, n, step, lr, beta1, beta2, eps, weight_decay, s);
     return e == hipSuccess ? 0 : hip_fail(e, "adamw launch");
+}
+
+namespace {
+int check_list(const void* ptrs, const long* numel, const long* chunk_start, int n, long chunks, int dtype) {
+    if (!ptrs || !numel || !chunk_start) return fail(MUON_HIP_EINVAL, "null tensor-list array");
+    if (n <= 0 || chunks <= 0) return fail(MUON_HIP_EINVAL, "a tensor list needs at least one tensor and one chunk");
+    if (chunks > 0x7fffffffL) return fail(MUON_HIP_ESHAPE, "%ld chunks exceed one launch", chunks);
+    if (!dtype_ok(dtype)) return fail(MUON_HIP_EINVAL, "unknown dtype %d", dtype);
+    return 0;
+}
+}  // namespace
+
+int muon_hip_adamw_multi(const void* const* p_ptrs, const void* const* g_ptrs, const void* const* exp_avg_ptrs,
+                         const void* const* exp_avg_sq_ptrs, const long* numel, const long* chunk_start,
+                         const double* bias1, const double* bias2, int n, long chunks, int dtype, double lr,
+                         double beta1, double beta2, double eps, double weight_decay, void* stream) {
+    if (int rc = check_list(p_ptrs, numel, chunk_start, n, chunks, dtype)) return rc;
+    if (!g_ptrs || !exp_avg_ptrs || !exp_avg_sq_ptrs || !bias1 || !bias2) return fail(MUON_HIP_EINVAL, "null table");
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_ADAMW_MULTI, s);
+    const MultiTensorList l{p_ptrs, numel, chunk_start, n, chunks};
+    hipError_t e = launch_adamw_multi(l, g_ptrs, exp_avg_ptrs, exp_avg_sq_ptrs, bias1, bias2, dtype, lr, beta1, beta2,
+                                      eps, weight_decay, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "adamw_multi launch");
+}
+
+int muon_hip_grad_norms(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
+                        int dtype, float* partials, float* norms, void* stream) {
+    if (int rc = check_list(g_ptrs, numel, chunk_start, n, chunks, dtype)) return rc;
+    if (!partials || !norms) return fail(MUON_HIP_EINVAL, "null output");
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_GRAD_NORM, s);
+    const MultiTensorList l{g_ptrs, numel, chunk_start, n, chunks};
+    hipError_t e = launch_tensor_norms(l, dtype, partials, norms, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "grad_norms launch");
+}
+
+int muon_hip_total_norm(const float* norms, int n, int dtype, float* total_f32, void* total_typed, void* stream) {
+    if (!norms || !total_f32 || !total_typed || n <= 0 || !dtype_ok(dtype))
+        return fail(MUON_HIP_EINVAL, "null pointer, empty list or unknown dtype");
+    hipError_t e = launch_total_norm(norms, n, dtype, total_f32, total_typed, (hipStream_t)stream);
+    return e == hipSuccess ? 0 : hip_fail(e, "total_norm launch");
+}
+
+int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
+                        int dtype, const float* total_f32, int norm_dtype, double max_norm, void* stream) {
+    if (int rc = check_list(g_ptrs, numel, chunk_start, n, chunks, dtype)) return rc;
+    if (!total_f32 || !dtype_ok(norm_dtype)) return fail(MUON_HIP_EINVAL, "null total or unknown norm dtype");
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_CLIP_SCALE, s);
+    const MultiTensorList l{g_ptrs, numel, chunk_start, n, chunks};
+    hipError_t e = launch_clip_scale_multi(l, dtype, total_f32, norm_dtype, max_norm, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "clip_scale launch");
 }
 
 int muon_hip_timing_enable(int on) {

@@ -1171,7 +1171,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
 #ifdef EXPP_L1_HIT
         voff = lane * 16; base = (const char*)Pb;
 #endif
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+#ifndef EXPP_CACHE_BITS
+#define EXPP_CACHE_BITS ""
+#endif
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" EXPP_CACHE_BITS
                      :
                      : "s"(lds_byte), "v"(voff), "s"(base)
                      : "memory");

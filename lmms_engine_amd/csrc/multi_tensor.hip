@@ -1,0 +1,287 @@
+// Multi-tensor memory-bound kernels: one launch walks a whole list of tensors.
+//
+//   adamw_multi      : adam_update + the Adam branch of step_fsdp (muon_utils.py:178-183,
+//                      :468-477) for every tensor of a parameter group
+//   sqnorm / norms   : the 2-norm torch's _get_total_norm computes for
+//                      fsdp2_clip_grad_norm_ (utils/fsdp2_utils.py:234-255): per-tensor norms
+//                      rounded to the tensor dtype, then the norm of those norms
+//   clip_scale_multi : _clip_grads_with_norm_: g *= clamp(max_norm / (total + 1e-6), max=1)
+//
+// A tensor list is cut into chunks of MUON_MULTI_CHUNK elements; chunk_start[t] is the index of
+// tensor t's first chunk (chunk_start[n] = number of chunks = grid size).  A block finds its
+// tensor by bisection and handles one chunk: 16-byte vectors when every base pointer of the
+// tensor is 16-byte aligned, scalars otherwise and for the last few elements.
+#include "multi_tensor.h"
+
+namespace {
+
+template <typename T> struct Mt;
+template <> struct Mt<float> {
+    static __device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+        const f32x4 a = *(const f32x4*)p, b = *(const f32x4*)(p + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { v[i] = a[i]; v[4 + i] = b[i]; }
+    }
+    static __device__ __forceinline__ void store8(float* p, const float (&v)[8]) {
+        f32x4 a, b;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { a[i] = v[i]; b[i] = v[4 + i]; }
+        *(f32x4*)p = a;
+        *(f32x4*)(p + 4) = b;
+    }
+    static __device__ __forceinline__ float rnd(float x) { return x; }
+    static __device__ __forceinline__ float load(const float* p) { return *p; }
+    static __device__ __forceinline__ void store(float* p, float x) { *p = x; }
+};
+template <> struct Mt<bf16_t> {
+    static __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+        const bf16x8 a = *(const bf16x8*)p;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = bf2f(a[i]);
+    }
+    static __device__ __forceinline__ void store8(bf16_t* p, const float (&v)[8]) {
+        bf16x8 a;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] = f2bf(v[i]);
+        *(bf16x8*)p = a;
+    }
+    static __device__ __forceinline__ float rnd(float x) { return rbf(x); }
+    static __device__ __forceinline__ float load(const bf16_t* p) { return bf2f(*p); }
+    static __device__ __forceinline__ void store(bf16_t* p, float x) { *p = f2bf(x); }
+};
+
+__device__ __forceinline__ float rnd_dtype(float x, int dtype) { return dtype == MUON_HIP_BF16 ? rbf(x) : x; }
+
+// tensor index t with chunk_start[t] <= chunk < chunk_start[t + 1]
+__device__ __forceinline__ int find_tensor(const long* chunk_start, int n, long chunk) {
+    int lo = 0, hi = n - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (chunk_start[mid] <= chunk) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
+}
+
+struct ChunkRange {
+    int t;
+    long begin, len;  // element offset in the tensor, elements in this chunk
+};
+
+__device__ __forceinline__ ChunkRange my_chunk(const long* numel, const long* chunk_start, int n) {
+    ChunkRange r;
+    r.t = find_tensor(chunk_start, n, blockIdx.x);
+    r.begin = ((long)blockIdx.x - chunk_start[r.t]) * MUON_MULTI_CHUNK;
+    const long left = numel[r.t] - r.begin;
+    r.len = left < MUON_MULTI_CHUNK ? left : MUON_MULTI_CHUNK;
+    return r;
+}
+
+__device__ __forceinline__ float lerp_aten(float s, float e, float w, float wm1, bool small) {
+    const float d = e - s;
+    return small ? fmaf(w, d, s) : fmaf(wm1, d, e);
+}
+
+struct AdamConst {
+    float w1, w1m1, w2, w2m1, eps, decay, alpha;
+    bool small1, small2;
+};
+
+template <typename T>
+__device__ __forceinline__ void adam_one(float& p, float g, float& e1, float& e2, const AdamConst& am, float c1, float c2) {
+    const float a = Mt<T>::rnd(lerp_aten(e1, g, am.w1, am.w1m1, am.small1));
+    const float g2 = Mt<T>::rnd(g * g);
+    const float bb = Mt<T>::rnd(lerp_aten(e2, g2, am.w2, am.w2m1, am.small2));
+    e1 = a;
+    e2 = bb;
+    const float ac = Mt<T>::rnd(__fdiv_rn(a, c1));
+    const float bc = Mt<T>::rnd(__fdiv_rn(bb, c2));
+    const float den = Mt<T>::rnd(Mt<T>::rnd(__fsqrt_rn(bc)) + am.eps);
+    const float upd = Mt<T>::rnd(__fdiv_rn(ac, den));
+    const float pd = Mt<T>::rnd(p * am.decay);
+    p = fmaf(am.alpha, upd, pd);  // stored through Mt<T>::store*, which rounds
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+adamw_multi_kernel(const void* const* p_ptrs, const void* const* g_ptrs, const void* const* e1_ptrs,
+                   const void* const* e2_ptrs, const long* numel, const long* chunk_start, const double* bias1,
+                   const double* bias2, int n, AdamConst am) {
+    const ChunkRange r = my_chunk(numel, chunk_start, n);
+    T* p = (T*)p_ptrs[r.t] + r.begin;
+    const T* g = (const T*)g_ptrs[r.t] + r.begin;
+    T* e1 = (T*)e1_ptrs[r.t] + r.begin;
+    T* e2 = (T*)e2_ptrs[r.t] + r.begin;
+    const float c1 = (float)bias1[r.t], c2 = (float)bias2[r.t];
+    const bool vec = ((((uintptr_t)p) | ((uintptr_t)g) | ((uintptr_t)e1) | ((uintptr_t)e2)) & 15) == 0;
+    const long n8 = vec ? r.len / 8 : 0;
+    for (long i = threadIdx.x; i < n8; i += 256) {
+        float pv[8], gv[8], av[8], bv[8];
+        Mt<T>::load8(p + i * 8, pv);
+        Mt<T>::load8(g + i * 8, gv);
+        Mt<T>::load8(e1 + i * 8, av);
+        Mt<T>::load8(e2 + i * 8, bv);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) adam_one<T>(pv[k], gv[k], av[k], bv[k], am, c1, c2);
+        Mt<T>::store8(e1 + i * 8, av);
+        Mt<T>::store8(e2 + i * 8, bv);
+        Mt<T>::store8(p + i * 8, pv);
+    }
+    for (long i = n8 * 8 + threadIdx.x; i < r.len; i += 256) {
+        float pv = Mt<T>::load(p + i), av = Mt<T>::load(e1 + i), bv = Mt<T>::load(e2 + i);
+        adam_one<T>(pv, Mt<T>::load(g + i), av, bv, am, c1, c2);
+        Mt<T>::store(e1 + i, av);
+        Mt<T>::store(e2 + i, bv);
+        Mt<T>::store(p + i, pv);
+    }
+}
+
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+sqnorm_multi_kernel(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, float* partials) {
+    __shared__ float red[4];
+    const ChunkRange r = my_chunk(numel, chunk_start, n);
+    const T* g = (const T*)g_ptrs[r.t] + r.begin;
+    const bool vec = (((uintptr_t)g) & 15) == 0;
+    const long n8 = vec ? r.len / 8 : 0;
+    float ss = 0.f;
+    for (long i = threadIdx.x; i < n8; i += 256) {
+        float v[8];
+        Mt<T>::load8(g + i * 8, v);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) ss = fmaf(v[k], v[k], ss);
+    }
+    for (long i = n8 * 8 + threadIdx.x; i < r.len; i += 256) {
+        const float v = Mt<T>::load(g + i);
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum_256(ss, red);
+    if (threadIdx.x == 0) partials[blockIdx.x] = ss;
+}
+
+// One block per tensor: its partial sums in a fixed order -> norm, rounded to the tensor dtype.
+__global__ void __launch_bounds__(256)
+tensor_norm_kernel(const float* partials, const long* chunk_start, int dtype, float* norms) {
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    float ss = 0.f;
+    for (long c = chunk_start[t] + threadIdx.x; c < chunk_start[t + 1]; c += 256) ss += partials[c];
+    ss = block_sum_256(ss, red);
+    if (threadIdx.x == 0) norms[t] = rnd_dtype(__fsqrt_rn(ss), dtype);
+}
+
+// One block: norm of the per-tensor norms, rounded to the result dtype; written as fp32 (for the
+// scaling kernel) and in the result dtype (the tensor the caller returns).
+__global__ void __launch_bounds__(256)
+total_norm_kernel(const float* norms, int n, int dtype, float* total_f32, void* total_typed) {
+    __shared__ float red[4];
+    float ss = 0.f;
+    for (int t = threadIdx.x; t < n; t += 256) ss = fmaf(norms[t], norms[t], ss);
+    ss = block_sum_256(ss, red);
+    if (threadIdx.x == 0) {
+        const float tn = rnd_dtype(__fsqrt_rn(ss), dtype);
+        *total_f32 = tn;
+        if (dtype == MUON_HIP_BF16) *(bf16_t*)total_typed = f2bf(tn);
+        else *(float*)total_typed = tn;
+    }
+}
+
+// torch evaluates max_norm / (total + 1e-6) as (total + 1e-6).reciprocal() * max_norm, every
+// step rounded to the norm's dtype, then clamps at 1.
+__device__ __forceinline__ float clip_coef(float total, int norm_dtype, float max_norm) {
+    const float s = rnd_dtype(total + 1e-6f, norm_dtype);
+    const float r = rnd_dtype(__fdiv_rn(1.0f, s), norm_dtype);
+    const float c = rnd_dtype(r * max_norm, norm_dtype);
+    return c > 1.0f ? 1.0f : c;  // a NaN coefficient stays NaN, as torch.clamp leaves it
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+clip_scale_multi_kernel(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n,
+                        const float* total_f32, int norm_dtype, float max_norm) {
+    const float coef = clip_coef(*total_f32, norm_dtype, max_norm);
+    const ChunkRange r = my_chunk(numel, chunk_start, n);
+    T* g = (T*)g_ptrs[r.t] + r.begin;
+    const bool vec = (((uintptr_t)g) & 15) == 0;
+    const long n8 = vec ? r.len / 8 : 0;
+    for (long i = threadIdx.x; i < n8; i += 256) {
+        float v[8];
+        Mt<T>::load8(g + i * 8, v);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] *= coef;
+        Mt<T>::store8(g + i * 8, v);
+    }
+    for (long i = n8 * 8 + threadIdx.x; i < r.len; i += 256) Mt<T>::store(g + i, Mt<T>::load(g + i) * coef);
+}
+
+inline void lerp_consts(double weight, float& w, float& wm1, bool& small) {
+    w = (float)weight;
+    wm1 = w - 1.0f;
+    small = fabsf(w) < 0.5f;
+}
+
+}  // namespace
+
+hipError_t launch_adamw_multi(const MultiTensorList& l, const void* const* g_ptrs, const void* const* e1_ptrs,
+                              const void* const* e2_ptrs, const double* bias1, const double* bias2, int dtype,
+                              double lr, double b1, double b2, double eps, double wd, hipStream_t stream) {
+    AdamConst am;
+    lerp_consts(1.0 - b1, am.w1, am.w1m1, am.small1);
+    lerp_consts(1.0 - b2, am.w2, am.w2m1, am.small2);
+    am.eps = (float)eps;
+    am.decay = (float)(1.0 - lr * wd);
+    am.alpha = (float)(-lr);
+    dim3 grid((unsigned)l.chunks), block(256);
+    if (dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((adamw_multi_kernel<float>), grid, block, 0, stream, l.ptrs, g_ptrs, e1_ptrs, e2_ptrs, l.numel,
+                           l.chunk_start, bias1, bias2, l.n, am);
+    else if (dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((adamw_multi_kernel<bf16_t>), grid, block, 0, stream, l.ptrs, g_ptrs, e1_ptrs, e2_ptrs, l.numel,
+                           l.chunk_start, bias1, bias2, l.n, am);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_tensor_norms(const MultiTensorList& l, int dtype, float* partials, float* norms, hipStream_t stream) {
+    dim3 grid((unsigned)l.chunks), block(256);
+    if (dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((sqnorm_multi_kernel<float>), grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n, partials);
+    else if (dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((sqnorm_multi_kernel<bf16_t>), grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n, partials);
+    else
+        return hipErrorInvalidValue;
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(tensor_norm_kernel, dim3((unsigned)l.n), block, 0, stream, partials, l.chunk_start, dtype, norms);
+    return hipGetLastError();
+}
+
+hipError_t launch_total_norm(const float* norms, int n, int dtype, float* total_f32, void* total_typed,
+                             hipStream_t stream) {
+    hipLaunchKernelGGL(total_norm_kernel, dim3(1), dim3(256), 0, stream, norms, n, dtype, total_f32, total_typed);
+    return hipGetLastError();
+}
+
+hipError_t launch_clip_scale_multi(const MultiTensorList& l, int dtype, const float* total_f32, int norm_dtype,
+                                   double max_norm, hipStream_t stream) {
+    dim3 grid((unsigned)l.chunks), block(256);
+    if (dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((clip_scale_multi_kernel<float>), grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n,
+                           total_f32, norm_dtype, (float)max_norm);
+    else if (dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((clip_scale_multi_kernel<bf16_t>), grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n,
+                           total_f32, norm_dtype, (float)max_norm);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}

@@ -395,6 +395,7 @@ class Muon(torch.optim.Optimizer):
                     _muon_bucket_step(ps, gs, ms, group, ns_steps, nesterov, self.write_back_grad, self._workspaces,
                                       self.workspace_limit_bytes)
             else:
+                items = []
                 for p in group["params"]:
                     if p.grad is None:
                         p.grad = torch.zeros_like(p)
@@ -404,12 +405,47 @@ class Muon(torch.optim.Optimizer):
                         state["exp_avg_sq"] = torch.zeros_like(p)
                         state["step"] = 0
                     state["step"] += 1
-                    _adamw_tensor(p, p.grad, state["exp_avg"], state["exp_avg_sq"], state["step"], group)
+                    items.append((p, p.grad, state["exp_avg"], state["exp_avg_sq"], state["step"]))
+                _adamw_group(items, group)
 
         for work in dq:
             work.finish()
 
         return loss
+
+
+def _adamw_group(items, group: dict) -> None:
+    """The Adam branch of step_fsdp (muon_utils.py:458-477) for a whole parameter group: one launch per
+    (device, dtype) over all its tensors.  Every parameter carries its own step, so the two bias
+    corrections travel as per-tensor doubles."""
+    from .multi_tensor import TensorListTable
+
+    buckets: "OrderedDict[tuple, list]" = OrderedDict()
+    for p, grad, e1, e2, step in items:
+        _require_cuda(p, "an AdamW parameter")
+        if not (p.is_contiguous() and e1.is_contiguous() and e2.is_contiguous()):
+            raise NotImplementedError("AdamW-fallback parameters and state must be contiguous")
+        if e1.dtype != p.dtype or e2.dtype != p.dtype:
+            raise NotImplementedError("AdamW-fallback state must have the parameter's dtype")
+        if p.numel() == 0:
+            continue
+        g = grad
+        if g.dtype != p.dtype or not g.is_contiguous():
+            g = g.to(p.dtype).contiguous()
+        buckets.setdefault((p.device, p.dtype), []).append((p, g, e1, e2, step))
+    b1, b2 = float(group["betas"][0]), float(group["betas"][1])
+    for (dev, dt), its in buckets.items():
+        ps, gs, e1s, e2s, steps = (list(t) for t in zip(*its))
+        with torch.cuda.device(dev):
+            tab = TensorListTable([ps, gs, e1s, e2s], doubles=[[1 - b1 ** st for st in steps], [1 - b2 ** st for st in steps]])
+            _abi.check(
+                _abi.lib().muon_hip_adamw_multi(
+                    *tab.role_ptrs, tab.numel_ptr, tab.chunk_start_ptr, *tab.double_ptrs, tab.n, tab.chunks,
+                    _abi.dtype_code(dt), float(group["lr"]), b1, b2, float(group["eps"]), float(group["weight_decay"]),
+                    _abi.stream_ptr(dev),
+                ),
+                "adamw_multi",
+            )
 
 
 def _adamw_tensor(p: Tensor, grad: Tensor, exp_avg: Tensor, exp_avg_sq: Tensor, step: int, group: dict) -> None:
