@@ -18,7 +18,7 @@
  *    K = max(rows, cols); "transposed" means rows > cols (muon_utils.py:139-140).
  *  - Batched entry points work on `batch` matrices of one shape.  Optimizer tensors are
  *    reached through device-resident pointer tables (`const void* const*`, `batch` entries).
- *  - The Newton-Schulz operands live in a caller-allocated workspace of
+ *  - The Newton-Schulz operands live, in a blocked layout (below), in a caller-allocated workspace of
  *    muon_hip_workspace_bytes() bytes, 256-byte aligned, which the entry points partition
  *    identically; its contents between calls are private to the library.
  */
@@ -50,27 +50,15 @@ extern "C" {
 #define MUON_HIP_K_CLIP_SCALE 9
 #define MUON_HIP_K_COUNT 10
 
-/* GEMM tile configurations; MUON_HIP_CFG_AUTO picks by shape. */
+/* GEMM kernel variants; MUON_HIP_CFG_AUTO picks per kernel and shape.  All feed LDS with direct
+ * global->LDS loads (global_load_lds_dwordx4), software pipelined behind the MFMAs. */
 #define MUON_HIP_CFG_AUTO (-1)
-#define MUON_HIP_CFG_128x128_W4 0
-#define MUON_HIP_CFG_256x256_W4 1
-#define MUON_HIP_CFG_256x256_W8 2
-/* the same tiles fed by direct global->LDS loads (global_load_lds_dwordx4) */
-#define MUON_HIP_CFG_128x128_W4_DLDS 3
-#define MUON_HIP_CFG_256x256_W4_DLDS 4
-#define MUON_HIP_CFG_256x256_W8_DLDS 5
-/* direct loads, software pipelined: MFMAs interleaved with LDS reads and loads, one barrier per k-tile */
-#define MUON_HIP_CFG_128x128_W4_PIPE 6
-#define MUON_HIP_CFG_256x256_W4_PIPE 7
-#define MUON_HIP_CFG_256x256_W8_PIPE 8
-/* 32-column k-tiles in four LDS stages: loads spread evenly between the MFMAs */
-#define MUON_HIP_CFG_128x128_W4_PIPE4 9
-#define MUON_HIP_CFG_256x256_W4_PIPE4 10
-#define MUON_HIP_CFG_256x256_W8_PIPE4 11
-/* two groups of four waves alternating between a memory phase and an MFMA-only phase */
-#define MUON_HIP_CFG_256x256_W8_PINGPONG 12
-/* the same with five LDS stages (all 160 KB): loads stay in flight one k-tile longer */
-#define MUON_HIP_CFG_256x256_W8_PINGPONG5 13
+#define MUON_HIP_CFG_128_PIPE 0      /* 128x128 tile, 4 waves, 64-column k-tiles, two LDS stages */
+#define MUON_HIP_CFG_256_PIPE 1      /* 256x256 tile, 8 waves, the same pipeline */
+#define MUON_HIP_CFG_128_PIPE4 2     /* 128x128 tile, 4 waves, 32-column k-tiles, four LDS stages */
+#define MUON_HIP_CFG_256_W4_PIPE4 3  /* 256x256 tile, 4 waves of 128x128, four LDS stages */
+#define MUON_HIP_CFG_256_PINGPONG 4  /* 256x256 tile, two groups of 4 waves alternating memory / MFMA phases */
+#define MUON_HIP_CFG_COUNT 5
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);
@@ -127,26 +115,36 @@ int muon_hip_step_grouped(const void* const* p_ptrs, const void* const* g_ptrs, 
                           double lr, double weight_decay, double beta, int nesterov, int ns_steps, double scale,
                           double a, double b, double c, int write_back_grad, void* stream);
 
-/* ---- single GEMM entry points (explicit buffers, already padded to whole tiles) -------
- * Every matrix is row-major with a row pitch `ld*` in elements (>= its width, a multiple of
- * 8); matrix b of a batch starts at b * rows * ld.  Pitches that are multiples of 2048
- * elements are legal but slow (all rows of a tile share an L2 channel): add 128. */
+/* ---- blocked matrices and single GEMM entry points ---------------------------------------
+ * The Newton-Schulz operands are kept in blocks of 256 rows x 32 columns (16 KB, 64-byte
+ * rows back to back): element (r, c) of a matrix with cb = cols / 32 column blocks is at
+ *     ((r / 256) * cb + c / 32) * 8192 + (r % 256) * 32 + c % 32
+ * so that every 32-column k-tile of an operand panel is one contiguous run of memory.  A blocked
+ * rows x cols matrix (cols a multiple of 32) takes muon_hip_blocked_elems(rows, cols) elements;
+ * matrix b of a batch starts b times that many elements after the first. */
+long muon_hip_blocked_elems(int rows, int cols);
 
-/* A[batch][Mp][lda] = bf16(X Xt) for X[batch][Mp][ldx] (Kp columns used):
- * matmul_transpose_assign + mmt_kernel, muon_utils.py:95-119 and :28-92.  Upper tiles
- * computed, mirrored below the diagonal. */
-int muon_hip_syrk_bf16(const void* X, int ldx, void* A, int lda, int Mp, int Kp, int batch, int cfg, void* stream);
+/* Row-major bf16 (row pitch ld, matrices src_stride elements apart) -> blocked rows_p x cols_p,
+ * zero padded; and back (only rows x cols are written). */
+int muon_hip_pack_bf16(const void* src, long src_stride, int ld, int rows, int cols, void* dst, int rows_p, int cols_p,
+                       int batch, void* stream);
+int muon_hip_unpack_bf16(const void* src, int rows_p, int cols_p, void* dst, long dst_stride, int ld, int rows, int cols,
+                         int batch, void* stream);
 
-/* B = bf16(bf16(b*A) + bf16(c*bf16(A A))) for symmetric A: muon_utils.py:150-151.
- * A and B share the pitch lda. */
-int muon_hip_sympoly_bf16(const void* A, void* B, int lda, int Mp, int batch, double b, double c, int cfg,
-                          void* stream);
+/* The three products on explicit blocked buffers already padded to whole tiles (Mp, Kp multiples
+ * of the configuration's tile edge). */
 
-/* X' = bf16(bf16(a*X) + bf16(B X)): muon_utils.py:152.  B[batch][Mp][lda] symmetric,
- * XT[batch][Kp][ldxt] the transposed copy of X; writes Xout[batch][Mp][ldx] and/or
- * XTout[batch][Kp][ldxt] (either may be null, not both). */
-int muon_hip_bx_axpy_bf16(const void* B, int lda, const void* XT, int ldxt, void* Xout, int ldx, void* XTout, int Mp,
-                          int Kp, int batch, double a, int cfg, void* stream);
+/* A (Mp x Mp) = bf16(X Xt) for X (Mp x Kp): matmul_transpose_assign + mmt_kernel,
+ * muon_utils.py:95-119 and :28-92.  Upper tiles computed, mirrored below the diagonal. */
+int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* stream);
+
+/* B = bf16(bf16(b*A) + bf16(c*bf16(A A))) for symmetric A (Mp x Mp): muon_utils.py:150-151. */
+int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* stream);
+
+/* X' = bf16(bf16(a*X) + bf16(B X)): muon_utils.py:152.  B (Mp x Mp) symmetric, XT (Kp x Mp) the
+ * transposed copy of X; writes Xout (Mp x Kp) and/or XTout (Kp x Mp) (either may be null, not both). */
+int muon_hip_bx_axpy_bf16(const void* B, const void* XT, void* Xout, void* XTout, int Mp, int Kp, int batch, double a,
+                          int cfg, void* stream);
 
 /* ---- AdamW fallback ------------------------------------------------------------------ */
 

@@ -15,12 +15,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmuon_hip.so")
 
 F32, BF16 = 0, 1
-CFG_AUTO, CFG_128x128_W4, CFG_256x256_W4, CFG_256x256_W8 = -1, 0, 1, 2
-CFG_128x128_W4_DLDS, CFG_256x256_W4_DLDS, CFG_256x256_W8_DLDS = 3, 4, 5
-CFG_128x128_W4_PIPE, CFG_256x256_W4_PIPE, CFG_256x256_W8_PIPE = 6, 7, 8
-CFG_128x128_W4_PIPE4, CFG_256x256_W4_PIPE4, CFG_256x256_W8_PIPE4 = 9, 10, 11
-CFG_256x256_W8_PINGPONG, CFG_256x256_W8_PINGPONG5 = 12, 13
-GEMM_CONFIGS = list(range(14))
+CFG_AUTO, CFG_128_PIPE, CFG_256_PIPE, CFG_128_PIPE4, CFG_256_W4_PIPE4, CFG_256_PINGPONG = -1, 0, 1, 2, 3, 4
+GEMM_CONFIGS = list(range(5))
 K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW, K_ADAMW_MULTI, K_GRAD_NORM, K_CLIP_SCALE = range(10)
 KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw", "adamw_multi",
                 "grad_norm", "clip_scale"]
@@ -43,10 +39,13 @@ SIGNATURES = {
     "muon_hip_step_grouped": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int,
                                       c_double, c_double, c_double, c_int, c_int, c_double, c_double, c_double,
                                       c_double, c_int, c_void_p]),
-    "muon_hip_syrk_bf16": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
-    "muon_hip_sympoly_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_double, c_int, c_void_p]),
-    "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int,
-                                      c_double, c_int, c_void_p]),
+    "muon_hip_blocked_elems": (c_long, [c_int, c_int]),
+    "muon_hip_pack_bf16": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "muon_hip_unpack_bf16": (c_int, [c_void_p, c_int, c_int, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p]),
+    "muon_hip_syrk_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "muon_hip_sympoly_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_double, c_double, c_int, c_void_p]),
+    "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_int,
+                                      c_void_p]),
     "muon_hip_adamw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_double,
                                c_double, c_double, c_double, c_void_p]),
     "muon_hip_adamw_multi": (c_int, [c_void_p] * 8 + [c_int, c_long, c_int] + [c_double] * 5 + [c_void_p]),

@@ -75,28 +75,23 @@ struct Timed {
 // ---- geometry / workspace ------------------------------------------------------------
 struct Plan {
     int rows, cols, batch, M, K, Mp, Kp, tile, cfg, nparts;
-    int ldx, ldxt, lda;  // row pitches (elements) of X, Xt and A/B
     bool transposed;
-    long n, strideU, strideX, strideXT, strideA;
+    long n, strideU, strideX, strideXT, strideA;  // elements per matrix: U dense, the others blocked
     size_t offX[2], offXT[2], offA, offB, offParts, offDenom, total;
 };
-
-constexpr int MUON_LD_PAD = 128;  // bf16 elements = 256 bytes
 
 inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
 
 // Tile edge for a matrix whose short side is M: 256 when M is a whole number of 256-tiles.
 bool use_tile256(int M) { return M % 256 == 0 && M >= 512; }
 
-// Configuration per kernel, from a sweep of every variant over the benchmark shapes.
-int pick_cfg(int M, int epi = EPI_BX) {
+// Configuration per kernel, from a sweep of every variant over the benchmark shapes: the ping-pong
+// kernel wherever 256-tiles fill the machine, 128-tiles for the symmetric products of small matrices.
+int pick_cfg(int M, int epi = EPI_BX, int kdim = 0) {
     if (g_forced_cfg != MUON_HIP_CFG_AUTO) return g_forced_cfg;
-    if (!use_tile256(M)) return epi == EPI_BX ? GEMM_CFG_128x128_W4_PIPE : GEMM_CFG_128x128_W4_PIPE4;
-    switch (epi) {
-        case EPI_SYRK: return M >= 1024 ? GEMM_CFG_256x256_W4_PIPE4 : GEMM_CFG_256x256_W8_PIPE;
-        case EPI_SYMPOLY: return M <= 1024 ? GEMM_CFG_128x128_W4_PIPE : GEMM_CFG_256x256_W8_PIPE;
-        default: return GEMM_CFG_256x256_W8_PIPE;
-    }
+    if (!use_tile256(M)) return (epi == EPI_SYRK && kdim < 2048) ? GEMM_CFG_128_PIPE4 : GEMM_CFG_128_PIPE;
+    if (epi != EPI_BX && M <= 512) return GEMM_CFG_128_PIPE;
+    return GEMM_CFG_256_PINGPONG;
 }
 
 int make_plan(int rows, int cols, int batch, Plan& p) {
@@ -115,15 +110,9 @@ int make_plan(int rows, int cols, int batch, Plan& p) {
     p.Kp = (int)round_up(p.K, p.tile);
     p.n = (long)rows * cols;
     p.strideU = round_up(p.n, 8);
-    // Row pitches that are multiples of 4 KB make every row of a tile land on the same L2
-    // channel (measured: 7 TB/s instead of 29 TB/s for L2-resident tiles); 256 bytes of
-    // padding per row spreads them.
-    p.ldx = p.Kp + MUON_LD_PAD;
-    p.ldxt = p.Mp + MUON_LD_PAD;
-    p.lda = p.Mp + MUON_LD_PAD;
-    p.strideX = (long)p.Mp * p.ldx;
-    p.strideXT = (long)p.Kp * p.ldxt;
-    p.strideA = (long)p.Mp * p.lda;
+    p.strideX = blocked_elems(p.Mp, p.Kp);
+    p.strideXT = blocked_elems(p.Kp, p.Mp);
+    p.strideA = blocked_elems(p.Mp, p.Mp);
     p.nparts = momentum_parts(p.n);
     const long T = p.Mp / p.tile, TN = p.Kp / p.tile;
     if (T * TN * batch > 0x7fffffffL) return fail(MUON_HIP_ESHAPE, "too many tiles for one launch");
@@ -155,11 +144,6 @@ int check_ws(const void* ws) {
     return 0;
 }
 
-int check_ld(int ld, int need, const char* what) {
-    if (ld < need || (ld % 8)) return fail(MUON_HIP_ESHAPE, "%s=%d must be >= %d and a multiple of 8 elements", what, ld, need);
-    return 0;
-}
-
 int check_gemm(int cfg, int Mp, int Kp, int batch, int& tile) {
     tile = gemm_cfg_tile(cfg);
     if (tile == 0) return fail(MUON_HIP_EINVAL, "unknown GEMM configuration %d", cfg);
@@ -170,40 +154,39 @@ int check_gemm(int cfg, int Mp, int Kp, int batch, int& tile) {
     return 0;
 }
 
-int do_syrk(int cfg, const bf16_t* X, int ldx, bf16_t* A, int lda, int Mp, int Kp, int batch, hipStream_t s) {
+// The three products on blocked buffers; matrix b of a batch starts at b * blocked_elems(rows, cols).
+int do_syrk(int cfg, const bf16_t* X, bf16_t* A, int Mp, int Kp, int batch, hipStream_t s) {
     GemmArgs g = {};
     const int tile = gemm_cfg_tile(cfg), T = Mp / tile;
     g.P = g.Q = X;
-    g.strideP = g.strideQ = (long)Mp * ldx;
-    g.ldp = g.ldq = ldx;
+    g.strideP = g.strideQ = blocked_elems(Mp, Kp);
     g.kdim = Kp;
     g.tiles_m = g.tiles_n = T;
     g.tiles_per_mat = T * (T + 1) / 2;
     g.batch = batch;
     g.C = g.Ct = A;
-    g.strideC = g.strideCt = (long)Mp * lda;
-    g.ldc = g.ldct = lda;
+    g.strideC = g.strideCt = blocked_elems(Mp, Mp);
+    g.cbC = g.cbCt = Mp / BLK_COLS;
     Timed t(MUON_HIP_K_SYRK, s);
     hipError_t e = launch_gemm_nt(cfg, EPI_SYRK, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "syrk launch");
 }
 
-int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int lda, int Mp, int batch, double b, double c, hipStream_t s) {
+int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b, double c, hipStream_t s) {
     GemmArgs g = {};
     const int tile = gemm_cfg_tile(cfg), T = Mp / tile;
     g.P = g.Q = A;
-    g.strideP = g.strideQ = (long)Mp * lda;
-    g.ldp = g.ldq = lda;
+    g.strideP = g.strideQ = blocked_elems(Mp, Mp);
     g.kdim = Mp;
     g.tiles_m = g.tiles_n = T;
     g.tiles_per_mat = T * (T + 1) / 2;
     g.batch = batch;
     g.C = g.Ct = B;
-    g.strideC = g.strideCt = (long)Mp * lda;
-    g.ldc = g.ldct = lda;
+    g.strideC = g.strideCt = blocked_elems(Mp, Mp);
+    g.cbC = g.cbCt = Mp / BLK_COLS;
     g.Et = A;
-    g.strideEt = (long)Mp * lda;
-    g.ldet = lda;
+    g.strideEt = blocked_elems(Mp, Mp);
+    g.cbEt = Mp / BLK_COLS;
     g.s0 = (float)b;
     g.s1 = (float)c;
     Timed t(MUON_HIP_K_SYMPOLY, s);
@@ -211,30 +194,28 @@ int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int lda, int Mp, int batch, 
     return e == hipSuccess ? 0 : hip_fail(e, "sympoly launch");
 }
 
-int do_bx(int cfg, const bf16_t* B, int lda, const bf16_t* XT, int ldxt, bf16_t* Xout, int ldx, bf16_t* XTout, int Mp,
-          int Kp, int batch, double a, hipStream_t s) {
+int do_bx(int cfg, const bf16_t* B, const bf16_t* XT, bf16_t* Xout, bf16_t* XTout, int Mp, int Kp, int batch, double a,
+          hipStream_t s) {
     GemmArgs g = {};
     const int tile = gemm_cfg_tile(cfg);
     g.P = B;
-    g.strideP = (long)Mp * lda;
-    g.ldp = lda;
+    g.strideP = blocked_elems(Mp, Mp);
     g.Q = XT;
-    g.strideQ = (long)Kp * ldxt;
-    g.ldq = ldxt;
+    g.strideQ = blocked_elems(Kp, Mp);
     g.kdim = Mp;
     g.tiles_m = Mp / tile;
     g.tiles_n = Kp / tile;
     g.tiles_per_mat = g.tiles_m * g.tiles_n;
     g.batch = batch;
     g.C = Xout;
-    g.strideC = (long)Mp * ldx;
-    g.ldc = ldx;
+    g.strideC = blocked_elems(Mp, Kp);
+    g.cbC = Kp / BLK_COLS;
     g.Ct = XTout;
-    g.strideCt = (long)Kp * ldxt;
-    g.ldct = ldxt;
+    g.strideCt = blocked_elems(Kp, Mp);
+    g.cbCt = Mp / BLK_COLS;
     g.Et = XT;
-    g.strideEt = (long)Kp * ldxt;
-    g.ldet = ldxt;
+    g.strideEt = blocked_elems(Kp, Mp);
+    g.cbEt = Mp / BLK_COLS;
     g.s0 = (float)a;
     Timed t(MUON_HIP_K_BX, s);
     hipError_t e = launch_gemm_nt(cfg, EPI_BX, g, s);
@@ -318,19 +299,18 @@ int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int step
     {
         Timed t(MUON_HIP_K_NORMALIZE, s);
         hipError_t e = launch_normalize(X[1], p.strideU, (const float*)((char*)workspace + p.offParts), p.nparts,
-                                        (float*)((char*)workspace + p.offDenom), X[0], p.ldx, p.strideX, XT[0], p.ldxt,
-                                        p.strideXT, rows, cols, p.Mp, p.Kp, batch, s);
+                                        (float*)((char*)workspace + p.offDenom), X[0], p.strideX, XT[0], p.strideXT, rows,
+                                        cols, p.Mp, p.Kp, batch, s);
         if (e != hipSuccess) return hip_fail(e, "normalize launch");
     }
     int cur = 0;
     for (int it = 0; it < steps; ++it) {
         const bool last = it + 1 == steps;
-        if (int rc = do_syrk(pick_cfg(p.M, EPI_SYRK), X[cur], p.ldx, A, p.lda, p.Mp, p.Kp, batch, s)) return rc;
-        if (int rc = do_sympoly(pick_cfg(p.M, EPI_SYMPOLY), A, B, p.lda, p.Mp, batch, b, c, s)) return rc;
+        if (int rc = do_syrk(pick_cfg(p.M, EPI_SYRK, p.Kp), X[cur], A, p.Mp, p.Kp, batch, s)) return rc;
+        if (int rc = do_sympoly(pick_cfg(p.M, EPI_SYMPOLY), A, B, p.Mp, batch, b, c, s)) return rc;
         bf16_t* xo = (last && p.transposed) ? nullptr : X[cur ^ 1];
         bf16_t* xto = (last && !p.transposed) ? nullptr : XT[cur ^ 1];
-        if (int rc = do_bx(pick_cfg(p.M, EPI_BX), B, p.lda, XT[cur], p.ldxt, xo, p.ldx, xto, p.Mp, p.Kp, batch, a, s))
-            return rc;
+        if (int rc = do_bx(pick_cfg(p.M, EPI_BX), B, XT[cur], xo, xto, p.Mp, p.Kp, batch, a, s)) return rc;
         cur ^= 1;
     }
     return 0;
@@ -345,10 +325,10 @@ int muon_hip_apply_update(const void* const* p_ptrs, int p_dtype, void* workspac
     hipStream_t s = (hipStream_t)stream;
     const int cur = steps & 1;
     const bf16_t* O = wsp(workspace, p.transposed ? p.offXT[cur] : p.offX[cur]);
-    const int ldo = p.transposed ? p.ldxt : p.ldx;
+    const int cbo = (p.transposed ? p.Mp : p.Kp) / BLK_COLS;  // O is rows x cols in the parameter's orientation
     const long strideO = p.transposed ? p.strideXT : p.strideX;
     Timed t(MUON_HIP_K_UPDATE, s);
-    hipError_t e = launch_apply_update(p_ptrs, p_dtype, O, strideO, ldo, rows, cols, batch, scale, lr, weight_decay, s);
+    hipError_t e = launch_apply_update(p_ptrs, p_dtype, O, strideO, cbo, rows, cols, batch, scale, lr, weight_decay, s);
     return e == hipSuccess ? 0 : hip_fail(e, "apply_update launch");
 }
 
@@ -360,9 +340,9 @@ int muon_hip_ns_output(void* workspace, int rows, int cols, int batch, int steps
     hipStream_t s = (hipStream_t)stream;
     const int cur = steps & 1;
     const bf16_t* O = wsp(workspace, p.transposed ? p.offXT[cur] : p.offX[cur]);
-    const int ldo = p.transposed ? p.ldxt : p.ldx;
+    const int cbo = (p.transposed ? p.Mp : p.Kp) / BLK_COLS;
     const long strideO = p.transposed ? p.strideXT : p.strideX;
-    hipError_t e = launch_gather_output((bf16_t*)out, p.n, O, strideO, ldo, rows, cols, batch, s);
+    hipError_t e = launch_unpack((bf16_t*)out, p.n, cols, O, strideO, cbo, rows, cols, batch, s);
     return e == hipSuccess ? 0 : hip_fail(e, "ns_output launch");
 }
 
@@ -378,38 +358,59 @@ int muon_hip_step_grouped(const void* const* p_ptrs, const void* const* g_ptrs, 
                                  stream);
 }
 
-int muon_hip_syrk_bf16(const void* X, int ldx, void* A, int lda, int Mp, int Kp, int batch, int cfg, void* stream) {
-    if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp, EPI_SYRK);
-    int tile;
-    if (int rc = check_gemm(cfg, Mp, Kp, batch, tile)) return rc;
-    if (int rc = check_ld(ldx, Kp, "ldx")) return rc;
-    if (int rc = check_ld(lda, Mp, "lda")) return rc;
-    if (!X || !A) return fail(MUON_HIP_EINVAL, "null operand");
-    return do_syrk(cfg, (const bf16_t*)X, ldx, (bf16_t*)A, lda, Mp, Kp, batch, (hipStream_t)stream);
+long muon_hip_blocked_elems(int rows, int cols) {
+    if (rows <= 0 || cols <= 0 || cols % BLK_COLS) {
+        fail(MUON_HIP_ESHAPE, "a blocked matrix needs positive sizes and a multiple of 32 columns (got %d x %d)", rows, cols);
+        return 0;
+    }
+    return blocked_elems(rows, cols);
 }
 
-int muon_hip_sympoly_bf16(const void* A, void* B, int lda, int Mp, int batch, double b, double c, int cfg,
-                          void* stream) {
+int muon_hip_pack_bf16(const void* src, long src_stride, int ld, int rows, int cols, void* dst, int rows_p, int cols_p,
+                       int batch, void* stream) {
+    if (!src || !dst || batch <= 0) return fail(MUON_HIP_EINVAL, "null tensor or empty batch");
+    if (rows <= 0 || cols <= 0 || rows > rows_p || cols > cols_p || ld < cols || cols_p % BLK_COLS || batch > 65535)
+        return fail(MUON_HIP_ESHAPE, "pack: need 0 < rows <= rows_p, 0 < cols <= cols_p, ld >= cols, cols_p %% 32 == 0");
+    hipError_t e = launch_pack((const bf16_t*)src, src_stride, ld, rows, cols, (bf16_t*)dst, blocked_elems(rows_p, cols_p),
+                               rows_p, cols_p, batch, (hipStream_t)stream);
+    return e == hipSuccess ? 0 : hip_fail(e, "pack launch");
+}
+
+int muon_hip_unpack_bf16(const void* src, int rows_p, int cols_p, void* dst, long dst_stride, int ld, int rows, int cols,
+                         int batch, void* stream) {
+    if (!src || !dst || batch <= 0) return fail(MUON_HIP_EINVAL, "null tensor or empty batch");
+    if (rows <= 0 || cols <= 0 || rows > rows_p || cols > cols_p || ld < cols || cols_p % BLK_COLS || batch > 65535)
+        return fail(MUON_HIP_ESHAPE, "unpack: need 0 < rows <= rows_p, 0 < cols <= cols_p, ld >= cols, cols_p %% 32 == 0");
+    hipError_t e = launch_unpack((bf16_t*)dst, dst_stride, ld, (const bf16_t*)src, blocked_elems(rows_p, cols_p),
+                                 cols_p / BLK_COLS, rows, cols, batch, (hipStream_t)stream);
+    return e == hipSuccess ? 0 : hip_fail(e, "unpack launch");
+}
+
+int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* stream) {
+    if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp, EPI_SYRK, Kp);
+    int tile;
+    if (int rc = check_gemm(cfg, Mp, Kp, batch, tile)) return rc;
+    if (!X || !A) return fail(MUON_HIP_EINVAL, "null operand");
+    return do_syrk(cfg, (const bf16_t*)X, (bf16_t*)A, Mp, Kp, batch, (hipStream_t)stream);
+}
+
+int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* stream) {
     if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp, EPI_SYMPOLY);
     int tile;
     if (int rc = check_gemm(cfg, Mp, Mp, batch, tile)) return rc;
-    if (int rc = check_ld(lda, Mp, "lda")) return rc;
     if (!A || !B || A == B) return fail(MUON_HIP_EINVAL, "null or aliased operand");
-    return do_sympoly(cfg, (const bf16_t*)A, (bf16_t*)B, lda, Mp, batch, b, c, (hipStream_t)stream);
+    return do_sympoly(cfg, (const bf16_t*)A, (bf16_t*)B, Mp, batch, b, c, (hipStream_t)stream);
 }
 
-int muon_hip_bx_axpy_bf16(const void* B, int lda, const void* XT, int ldxt, void* Xout, int ldx, void* XTout, int Mp,
-                          int Kp, int batch, double a, int cfg, void* stream) {
+int muon_hip_bx_axpy_bf16(const void* B, const void* XT, void* Xout, void* XTout, int Mp, int Kp, int batch, double a,
+                          int cfg, void* stream) {
     if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp, EPI_BX);
     int tile;
     if (int rc = check_gemm(cfg, Mp, Kp, batch, tile)) return rc;
-    if (int rc = check_ld(lda, Mp, "lda")) return rc;
-    if (int rc = check_ld(ldxt, Mp, "ldxt")) return rc;
-    if (int rc = check_ld(ldx, Kp, "ldx")) return rc;
     if (!B || !XT || (!Xout && !XTout)) return fail(MUON_HIP_EINVAL, "null operand");
     if (XTout == XT) return fail(MUON_HIP_EINVAL, "XTout must not alias XT");
-    return do_bx(cfg, (const bf16_t*)B, lda, (const bf16_t*)XT, ldxt, (bf16_t*)Xout, ldx, (bf16_t*)XTout, Mp, Kp, batch,
-                 a, (hipStream_t)stream);
+    return do_bx(cfg, (const bf16_t*)B, (const bf16_t*)XT, (bf16_t*)Xout, (bf16_t*)XTout, Mp, Kp, batch, a,
+                 (hipStream_t)stream);
 }
 
 int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int dtype, long n, int step, double lr,

@@ -17,6 +17,24 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define XCD_COUNT 8
 
+// Every matrix of the Newton-Schulz workspace is stored in blocks of 256 rows x BLK_COLS
+// columns (rows of a block back to back): element (r, c) of a matrix with `cb` column blocks is at
+//   ((r / 256) * cb + c / BLK_COLS) * BLK_ELEMS + (r % 256) * BLK_COLS + c % BLK_COLS.
+// A k-tile of an operand panel is then one contiguous run of memory instead of 256 row pieces
+// a row pitch apart, which is what DRAM pages, the L2 channels and the TLB all prefer.
+#ifndef MUON_BLK_COLS
+#define MUON_BLK_COLS 32
+#endif
+constexpr int BLK_ROWS = 256, BLK_COLS = MUON_BLK_COLS, BLK_SHIFT = BLK_COLS == 64 ? 6 : 5;
+constexpr int BLK_ELEMS = BLK_ROWS * BLK_COLS;
+static_assert(BLK_COLS == 32 || BLK_COLS == 64, "block width");
+
+__host__ __device__ inline long blocked_offset(long r, long c, int cb) {
+    return ((r >> 8) * cb + (c >> BLK_SHIFT)) * BLK_ELEMS + (r & 255) * BLK_COLS + (c & (BLK_COLS - 1));
+}
+// elements of a blocked rows x cols matrix (cols a multiple of BLK_COLS)
+inline long blocked_elems(long rows, long cols) { return ((rows + BLK_ROWS - 1) / BLK_ROWS) * (cols / BLK_COLS) * BLK_ELEMS; }
+
 // fp32 -> bf16, round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950), and back.
 __device__ __forceinline__ bf16_t f2bf(float f) { return (bf16_t)f; }
 __device__ __forceinline__ float bf2f(bf16_t h) { return (float)h; }

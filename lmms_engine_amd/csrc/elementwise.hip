@@ -188,22 +188,23 @@ __global__ void __launch_bounds__(256) frob_finalize_kernel(const float* partial
 }
 
 // One 64x128 tile of the bf16 blend u (parameter layout, rows x cols) divided by d, written
-// into the padded operand that has u's orientation (256-byte row segments) and, through an LDS
-// transpose, into the other one (128-byte row segments).  X is M x K, Xt is K x M.
+// into the blocked operand that has u's orientation and, through an LDS transpose, into the other
+// one; both leave as 128-byte row pieces that are neighbours inside a 256x64 block (2 KB and 4 KB
+// contiguous per pass).  X is M x K, Xt is K x M, both zero padded to Mp x Kp / Kp x Mp.
 __global__ void __launch_bounds__(256)
-normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, int ldx, long strideX, bf16_t* XT,
-                 int ldxt, long strideXT, int rows, int cols, int Mp, int Kp) {
+normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, long strideX, bf16_t* XT,
+                 long strideXT, int rows, int cols, int Mp, int Kp) {
     constexpr int TR = 64, TC = 128, PITCH = TC + 8;
     __shared__ __align__(16) bf16_t tile[TR][PITCH];
     const int b = blockIdx.y;
     const float d = denom[b];
     const bf16_t* u = U + b * strideU;
-    // transposed (rows > cols): X = u^T, so the padded row-major image of u is Xt.
+    // transposed (rows > cols): X = u^T, so the padded image of u is Xt.
     const bool transposed = rows > cols;
-    const int Cp = transposed ? Mp : Kp;                                  // padded cols of u's image
+    const int Cp = transposed ? Mp : Kp, Rp = transposed ? Kp : Mp;       // padded cols / rows of u's image
     bf16_t* same = transposed ? XT + b * strideXT : X + b * strideX;      // same orientation as u
     bf16_t* flip = transposed ? X + b * strideX : XT + b * strideXT;      // the transposed image
-    const int ld_same = transposed ? ldxt : ldx, ld_flip = transposed ? ldx : ldxt;
+    const int cb_same = Cp / BLK_COLS, cb_flip = Rp / BLK_COLS;
     const int tiles_c = Cp / TC;
     const int r0 = (blockIdx.x / tiles_c) * TR, c0 = (blockIdx.x % tiles_c) * TC;
     const int tr = threadIdx.x >> 4, tc = (threadIdx.x & 15) * 8;  // 16 rows x 16 chunks per pass
@@ -226,7 +227,7 @@ normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, i
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[i] = f2bf(__fdiv_rn(bf2f(v[h][i]), d));
         *(bf16x8*)(&tile[tr + h * 16][tc]) = o;
-        *(bf16x8*)(same + (long)r * ld_same + c) = o;
+        *(bf16x8*)(same + blocked_offset(r, c, cb_same)) = o;
     }
     __syncthreads();
     // flip[c][r]: 128 rows of 64 elements; a thread gathers 8 consecutive r of one column
@@ -237,7 +238,7 @@ normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, i
         bf16x8 o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[i] = tile[fr + i][fc];
-        *(bf16x8*)(flip + (long)(c0 + fc) * ld_flip + r0 + fr) = o;
+        *(bf16x8*)(flip + blocked_offset(c0 + fc, r0 + fr, cb_flip)) = o;
     }
 }
 
@@ -252,41 +253,45 @@ __device__ __forceinline__ float update_one(float p, float o, const UpdateMath& 
     return fmaf(um.alpha, os, pd);
 }
 
-// p <- p (1 - lr wd) - lr bf(O s); O is the NS output in the parameter's orientation with
-// a padded row stride.
+// p <- p (1 - lr wd) - lr bf(O s); O is the NS output in the parameter's orientation, blocked
+// with cbo column blocks.
 template <typename PT>
 __global__ void __launch_bounds__(256)
-apply_update_kernel(const void* const* p_ptrs, const bf16_t* O, long strideO, int ldo, int rows, int cols,
+apply_update_kernel(const void* const* p_ptrs, const bf16_t* O, long strideO, int cbo, int rows, int cols,
                     UpdateMath um) {
     const int b = blockIdx.y;
     PT* p = (PT*)p_ptrs[b];
     const bf16_t* o = O + b * strideO;
     const bool vec = (cols % 8 == 0) && ((((uintptr_t)p) & 15) == 0);
     if (vec) {
-        const int gpr = cols / 8;
-        const long n8 = (long)rows * gpr;
-        const long per_block = ((n8 + gridDim.x - 1) / gridDim.x + 511) / 512 * 512;
-        const long lo8 = (long)blockIdx.x * per_block, hi8 = lo8 + per_block < n8 ? lo8 + per_block : n8;
-        for (long i8 = lo8 + threadIdx.x; i8 < hi8; i8 += 512) {
-            const long j8 = i8 + 256;
-            const bool two = j8 < hi8;
+        // Tiles of 16 rows x 128 columns, a thread per 8 columns: in O a tile is four runs of 1 KB (16 rows of a
+        // column block lie back to back), in p sixteen row pieces that the next tile of the block continues.
+        const int tiles_c = (cols + 127) / 128;
+        const long ntiles = (long)((rows + 15) / 16) * tiles_c;
+        const long per_block = (ntiles + gridDim.x - 1) / gridDim.x;
+        const long t_lo = (long)blockIdx.x * per_block, t_hi = t_lo + per_block < ntiles ? t_lo + per_block : ntiles;
+        const int tr = threadIdx.x >> 4, tc = (threadIdx.x & 15) * 8;
+        for (long t = t_lo; t < t_hi; t += 2) {
             float pv[2][8], ov[2][8];
-            {
-                const long r = i8 / gpr;
-                Ld<PT>::template load8<true>(p + i8 * 8, pv[0]);
-                Ld<bf16_t>::template load8<true>(o + r * ldo + (int)(i8 - r * gpr) * 8, ov[0]);
-            }
-            if (two) {
-                const long r = j8 / gpr;
-                Ld<PT>::template load8<true>(p + j8 * 8, pv[1]);
-                Ld<bf16_t>::template load8<true>(o + r * ldo + (int)(j8 - r * gpr) * 8, ov[1]);
+            long off[2];
+            bool on[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const long tt = t + h;
+                const int r = (int)(tt / tiles_c) * 16 + tr, c = (int)(tt % tiles_c) * 128 + tc;
+                on[h] = tt < t_hi && r < rows && c < cols;
+                off[h] = (long)r * cols + c;
+                if (on[h]) {
+                    Ld<PT>::template load8<true>(p + off[h], pv[h]);
+                    Ld<bf16_t>::template load8<true>(o + blocked_offset(r, c, cbo), ov[h]);
+                }
             }
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                if (h == 1 && !two) break;
+                if (!on[h]) continue;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) pv[h][i] = update_one<PT>(pv[h][i], ov[h][i], um);
-                Ld<PT>::template store8<true>(p + (h ? j8 : i8) * 8, pv[h]);
+                Ld<PT>::template store8<true>(p + off[h], pv[h]);
             }
         }
     } else {
@@ -294,20 +299,39 @@ apply_update_kernel(const void* const* p_ptrs, const bf16_t* O, long strideO, in
         for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
             const long r = i / cols;
             const int c = (int)(i - r * cols);
-            Ld<PT>::store(p + i, update_one<PT>(Ld<PT>::load(p + i), bf2f(o[r * ldo + c]), um));
+            Ld<PT>::store(p + i, update_one<PT>(Ld<PT>::load(p + i), bf2f(o[blocked_offset(r, c, cbo)]), um));
         }
     }
 }
 
-// Scaled NS output into a dense (rows x cols) bf16 tensor: fast_newtonschulz called alone.
+// A blocked matrix into a dense row-major bf16 tensor (row pitch ld): the NS output of
+// fast_newtonschulz called alone, and the result of a single GEMM.
 __global__ void __launch_bounds__(256)
-gather_output_kernel(bf16_t* out, long strideOut, const bf16_t* O, long strideO, int ldo, int rows, int cols) {
+unpack_kernel(bf16_t* out, long strideOut, int ld, const bf16_t* O, long strideO, int cbo, int rows, int cols) {
     const int b = blockIdx.y;
     const long n = (long)rows * cols;
     for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
         const long r = i / cols;
         const int c = (int)(i - r * cols);
-        out[b * strideOut + i] = O[b * strideO + r * ldo + c];
+        out[b * strideOut + r * ld + c] = O[b * strideO + blocked_offset(r, c, cbo)];
+    }
+}
+
+// A dense row-major bf16 matrix (row pitch ld) into the blocked layout, zero padded to
+// rows_p x cols_p; one thread per 8 consecutive columns of the blocked image.
+__global__ void __launch_bounds__(256)
+pack_kernel(const bf16_t* src, long strideSrc, int ld, int rows, int cols, bf16_t* dst, long strideDst, int rows_p,
+            int cols_p) {
+    const int b = blockIdx.y;
+    const int cb = cols_p / BLK_COLS;
+    const long n8 = (long)rows_p * (cols_p / 8);
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n8; i += (long)gridDim.x * 256) {
+        const long r = i / (cols_p / 8);
+        const int c = (int)(i - r * (cols_p / 8)) * 8;
+        bf16x8 v;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = (r < rows && c + k < cols) ? src[b * strideSrc + r * ld + c + k] : (bf16_t)0.f;
+        *(bf16x8*)(dst + b * strideDst + blocked_offset(r, c, cb)) = v;
     }
 }
 
@@ -389,17 +413,17 @@ hipError_t launch_cast_norm(const void* G, long strideG, int g_dtype, bf16_t* U,
 }
 
 hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, float* denom, bf16_t* X,
-                            int ldx, long strideX, bf16_t* XT, int ldxt, long strideXT, int rows, int cols, int Mp,
-                            int Kp, int batch, hipStream_t stream) {
+                            long strideX, bf16_t* XT, long strideXT, int rows, int cols, int Mp, int Kp, int batch,
+                            hipStream_t stream) {
     hipLaunchKernelGGL(frob_finalize_kernel, dim3(batch), dim3(256), 0, stream, partials, nparts, denom);
     // u's padded image is Rp x Cp with Rp a multiple of 64 and Cp a multiple of 128 (both are multiples of the tile edge)
     dim3 grid((Mp / 64) * (Kp / 64) / 2, batch), block(256);
-    hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, ldx, strideX, XT, ldxt, strideXT,
-                       rows, cols, Mp, Kp);
+    hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, strideX, XT, strideXT, rows, cols,
+                       Mp, Kp);
     return hipGetLastError();
 }
 
-hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf16_t* O, long strideO, int ldo,
+hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf16_t* O, long strideO, int cbo,
                                int rows, int cols, int batch, double scale, double lr, double wd,
                                hipStream_t stream) {
     UpdateMath um;
@@ -408,19 +432,26 @@ hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf1
     um.alpha = (float)(-lr);
     dim3 grid(blocks_for((long)rows * cols, 16384, 8192), batch), block(256);
     if (p_dtype == MUON_HIP_F32)
-        hipLaunchKernelGGL((apply_update_kernel<float>), grid, block, 0, stream, p_ptrs, O, strideO, ldo, rows, cols, um);
+        hipLaunchKernelGGL((apply_update_kernel<float>), grid, block, 0, stream, p_ptrs, O, strideO, cbo, rows, cols, um);
     else if (p_dtype == MUON_HIP_BF16)
-        hipLaunchKernelGGL((apply_update_kernel<bf16_t>), grid, block, 0, stream, p_ptrs, O, strideO, ldo, rows, cols,
+        hipLaunchKernelGGL((apply_update_kernel<bf16_t>), grid, block, 0, stream, p_ptrs, O, strideO, cbo, rows, cols,
                            um);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();
 }
 
-hipError_t launch_gather_output(bf16_t* out, long strideOut, const bf16_t* O, long strideO, int ldo, int rows,
-                                int cols, int batch, hipStream_t stream) {
+hipError_t launch_unpack(bf16_t* out, long strideOut, int ld, const bf16_t* O, long strideO, int cbo, int rows,
+                         int cols, int batch, hipStream_t stream) {
     dim3 grid(blocks_for((long)rows * cols, 256 * 8, 2048), batch), block(256);
-    hipLaunchKernelGGL(gather_output_kernel, grid, block, 0, stream, out, strideOut, O, strideO, ldo, rows, cols);
+    hipLaunchKernelGGL(unpack_kernel, grid, block, 0, stream, out, strideOut, ld, O, strideO, cbo, rows, cols);
+    return hipGetLastError();
+}
+
+hipError_t launch_pack(const bf16_t* src, long strideSrc, int ld, int rows, int cols, bf16_t* dst, long strideDst,
+                       int rows_p, int cols_p, int batch, hipStream_t stream) {
+    dim3 grid(blocks_for((long)rows_p * cols_p / 8, 256 * 4, 4096), batch), block(256);
+    hipLaunchKernelGGL(pack_kernel, grid, block, 0, stream, src, strideSrc, ld, rows, cols, dst, strideDst, rows_p, cols_p);
     return hipGetLastError();
 }
 

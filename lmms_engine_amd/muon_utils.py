@@ -81,20 +81,21 @@ def matmul_transpose_assign(d_in: Tensor, d_out: Tensor) -> None:
     if d_in.dtype != torch.bfloat16:
         raise TypeError(f"the MI355X kernel multiplies bfloat16 operands, got {d_in.dtype}")
     M, K = d_in.shape
-    geo = _abi.geometry(M, max(K, M))  # tile choice follows the small side
-    tile = geo["tile"]
+    tile = 256 if (M % 256 == 0 and M >= 512) else 128
+    cfg = _abi.CFG_AUTO if tile == 256 else _abi.CFG_128_PIPE4
     Mp, Kp = -(-M // tile) * tile, -(-K // tile) * tile
-    ldx, lda = Kp + 128, Mp + 128  # padded pitches keep the rows of a tile on different L2 channels
+    lib = _abi.lib()
     with torch.cuda.device(d_in.device):
-        x = torch.zeros(Mp, ldx, dtype=torch.bfloat16, device=d_in.device)
-        x[:M, :K].copy_(d_in)
-        a = torch.empty(Mp, lda, dtype=torch.bfloat16, device=d_in.device)
-        _abi.check(
-            _abi.lib().muon_hip_syrk_bf16(x.data_ptr(), ldx, a.data_ptr(), lda, Mp, Kp, 1, _abi.CFG_AUTO,
-                                          _abi.stream_ptr(d_in.device)),
-            "syrk",
-        )
-        d_out.copy_(a[:M, :M])
+        s = _abi.stream_ptr(d_in.device)
+        src = d_in.contiguous()
+        x = torch.empty(lib.muon_hip_blocked_elems(Mp, Kp), dtype=torch.bfloat16, device=d_in.device)
+        a = torch.empty(lib.muon_hip_blocked_elems(Mp, Mp), dtype=torch.bfloat16, device=d_in.device)
+        _abi.check(lib.muon_hip_pack_bf16(src.data_ptr(), 0, K, M, K, x.data_ptr(), Mp, Kp, 1, s), "pack")
+        _abi.check(lib.muon_hip_syrk_bf16(x.data_ptr(), a.data_ptr(), Mp, Kp, 1, cfg, s), "syrk")
+        out = d_out if d_out.is_contiguous() else torch.empty_like(d_out, memory_format=torch.contiguous_format)
+        _abi.check(lib.muon_hip_unpack_bf16(a.data_ptr(), Mp, Mp, out.data_ptr(), 0, M, M, M, 1, s), "unpack")
+        if out is not d_out:
+            d_out.copy_(out)
 
 
 def matmul_transpose(d_in: Tensor) -> Tensor:

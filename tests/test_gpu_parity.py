@@ -47,7 +47,58 @@ def _assert_product_close(got, ref64, absprod):
     assert not bad.any(), f"{int(bad.sum())} elements outside one bf16 ulp"
 
 
-CFGS = list(range(14))
+CFGS = list(range(5))
+
+
+def _pack(env, t):
+    """[batch, rows, cols] bf16 on the device -> blocked buffer (shapes here are whole tiles already)."""
+    lib, abi = env["lib"], env["abi"]
+    batch, rows, cols = t.shape
+    t = t.contiguous()
+    out = torch.full((batch * lib.muon_hip_blocked_elems(rows, cols),), float("nan"), dtype=torch.bfloat16, device=t.device)
+    abi.check(lib.muon_hip_pack_bf16(t.data_ptr(), rows * cols, cols, rows, cols, out.data_ptr(), rows, cols, batch, 0))
+    return out
+
+
+def _blocked_nan(env, batch, rows, cols):
+    n = batch * env["lib"].muon_hip_blocked_elems(rows, cols)
+    return torch.full((n,), float("nan"), dtype=torch.bfloat16, device=env["dev"])
+
+
+def _unpack(env, buf, batch, rows, cols):
+    lib, abi = env["lib"], env["abi"]
+    out = torch.empty(batch, rows, cols, dtype=torch.bfloat16, device=buf.device)
+    abi.check(lib.muon_hip_unpack_bf16(buf.data_ptr(), rows, cols, out.data_ptr(), rows * cols, cols, rows, cols, batch, 0))
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def test_pack_unpack_round_trip_and_layout(env):
+    """The blocked layout is what include/muon_hip.h states: element (r, c) at
+    ((r/256)*cb + c/32)*8192 + (r%256)*32 + c%32, zero padded."""
+    lib, abi, dev = env["lib"], env["abi"], env["dev"]
+    g = torch.Generator().manual_seed(3)
+    rows, cols, rp, cp, batch = 300, 200, 384, 256, 2
+    t = torch.randn(batch, rows, cols + 8, generator=g).bfloat16().to(dev)  # row pitch 208 > cols
+    n = lib.muon_hip_blocked_elems(rp, cp)
+    assert n == 2 * 8 * 8192
+    buf = torch.full((batch * n,), float("nan"), dtype=torch.bfloat16, device=dev)
+    abi.check(lib.muon_hip_pack_bf16(t.data_ptr(), rows * (cols + 8), cols + 8, rows, cols, buf.data_ptr(), rp, cp, batch, 0))
+    torch.cuda.synchronize()
+    host, src = buf.cpu().view(batch, n), t.cpu()  # rows 384..511 of the last row of blocks are never touched
+    r = torch.arange(rp).view(-1, 1).expand(rp, cp)
+    c = torch.arange(cp).view(1, -1).expand(rp, cp)
+    idx = ((r // 256) * (cp // 32) + c // 32) * 8192 + (r % 256) * 32 + c % 32
+    for b in range(batch):
+        img = host[b][idx]
+        assert not torch.isnan(img).any()
+        assert torch.equal(img[:rows, :cols], src[b, :, :cols])
+        assert (img[rows:, :] == 0).all() and (img[:, cols:] == 0).all()
+    out = torch.full((batch, rows, cols + 3), 7.0, dtype=torch.bfloat16, device=dev)
+    abi.check(lib.muon_hip_unpack_bf16(buf.data_ptr(), rp, cp, out.data_ptr(), rows * (cols + 3), cols + 3, rows, cols, batch, 0))
+    torch.cuda.synchronize()
+    assert torch.equal(out.cpu()[:, :, :cols], src[:, :, :cols]) and (out.cpu()[:, :, cols:] == 7.0).all()
+    assert lib.muon_hip_blocked_elems(256, 100) == 0 and lib.muon_hip_pack_bf16(t.data_ptr(), 0, 8, 300, 200, buf.data_ptr(), rp, cp, 1, 0) == -2
 
 
 @pytest.mark.parametrize("cfg", CFGS)
@@ -56,11 +107,10 @@ def test_syrk_matches_fp64_and_is_symmetric(env, cfg, M, K, batch):
     print(f"syrk cfg={cfg} M={M} K={K} batch={batch}", flush=True)
     g = torch.Generator().manual_seed(10 + cfg)
     X = torch.randn(batch, M, K, generator=g).bfloat16()
-    Xd = X.to(env["dev"])
-    A = torch.full((batch, M, M), float("nan"), dtype=torch.bfloat16, device=env["dev"])
-    env["abi"].check(env["lib"].muon_hip_syrk_bf16(Xd.data_ptr(), K, A.data_ptr(), M, M, K, batch, cfg, 0))
-    torch.cuda.synchronize()
-    A = A.cpu()
+    Xb = _pack(env, X.to(env["dev"]))
+    Ab = _blocked_nan(env, batch, M, M)
+    env["abi"].check(env["lib"].muon_hip_syrk_bf16(Xb.data_ptr(), Ab.data_ptr(), M, K, batch, cfg, 0))
+    A = _unpack(env, Ab, batch, M, M)
     assert torch.equal(A, A.mT), "X·Xᵀ must be symmetric bit for bit"
     ref64 = (X.double() @ X.double().mT)
     _assert_product_close(A, ref64, X.double().abs() @ X.double().abs().mT)
@@ -75,12 +125,11 @@ def test_sympoly_rounding_points(env, cfg):
     M, batch = 512, 2
     X = (torch.randn(batch, M, 1024, generator=g) / 32).bfloat16()
     A = torch.stack([O.mmt(X[i]) for i in range(batch)])
-    Ad = A.to(env["dev"])
-    B = torch.full_like(Ad, float("nan"))
+    Ab = _pack(env, A.to(env["dev"]))
+    Bb = _blocked_nan(env, batch, M, M)
     a, b, c = O.NS_COEFFS
-    env["abi"].check(env["lib"].muon_hip_sympoly_bf16(Ad.data_ptr(), B.data_ptr(), M, M, batch, b, c, cfg, 0))
-    torch.cuda.synchronize()
-    B = B.cpu()
+    env["abi"].check(env["lib"].muon_hip_sympoly_bf16(Ab.data_ptr(), Bb.data_ptr(), M, batch, b, c, cfg, 0))
+    B = _unpack(env, Bb, batch, M, M)
     assert torch.equal(B, B.mT)
     for i in range(batch):
         A2 = O.mmt(A[i])
@@ -102,38 +151,42 @@ def test_bx_axpy_rounding_points(env, cfg, outputs):
     Bm = (torch.randn(batch, M, M, generator=g) / 16).bfloat16()
     Bm = torch.triu(Bm) + torch.triu(Bm, 1).mT  # the kernel is specified for symmetric B
     dev = env["dev"]
-    Xo = torch.full((batch, M, K), float("nan"), dtype=torch.bfloat16, device=dev)
-    XTo = torch.full((batch, K, M), float("nan"), dtype=torch.bfloat16, device=dev)
-    XT = X.mT.contiguous().to(dev)
+    Xo, XTo = _blocked_nan(env, batch, M, K), _blocked_nan(env, batch, K, M)
+    XT = _pack(env, X.mT.contiguous().to(dev))
+    Bb = _pack(env, Bm.to(dev))
     a = O.NS_COEFFS[0]
     env["abi"].check(env["lib"].muon_hip_bx_axpy_bf16(
-        Bm.to(dev).data_ptr(), M, XT.data_ptr(), M, Xo.data_ptr() if outputs != "xt" else None, K,
+        Bb.data_ptr(), XT.data_ptr(), Xo.data_ptr() if outputs != "xt" else None,
         XTo.data_ptr() if outputs != "x" else None, M, K, batch, a, cfg, 0))
-    torch.cuda.synchronize()
+    Xo, XTo = _unpack(env, Xo, batch, M, K), _unpack(env, XTo, batch, K, M)
     for i in range(batch):
         ref = (O.bf(X[i].float() * O._f32(a)) + O.bf(Bm[i].float() @ X[i].float())).bfloat16()
         if outputs != "xt":
-            got = Xo[i].cpu()
+            got = Xo[i]
             assert (got != ref).float().mean().item() < 2e-2
             assert rel_fro(got, ref) < 4e-3
+        else:
+            assert torch.isnan(Xo).all()
         if outputs != "x":
-            got = XTo[i].cpu().mT
+            got = XTo[i].mT
             assert (got != ref).float().mean().item() < 2e-2
             assert rel_fro(got, ref) < 4e-3
+        else:
+            assert torch.isnan(XTo).all()
     if outputs == "both":
-        assert torch.equal(Xo.cpu(), XTo.cpu().mT)
+        assert torch.equal(Xo, XTo.mT)
 
 
 def test_gemm_entry_points_reject_bad_shapes(env):
     lib, abi = env["lib"], env["abi"]
-    x = torch.zeros(256, 256, dtype=torch.bfloat16, device=env["dev"])
-    assert lib.muon_hip_syrk_bf16(x.data_ptr(), 256, x.data_ptr(), 256, 200, 256, 1, 0, 0) == -2
+    x = torch.zeros(256 * 256, dtype=torch.bfloat16, device=env["dev"])
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 200, 256, 1, 0, 0) == -2
     assert b"multiples" in lib.muon_hip_last_error()
-    assert lib.muon_hip_syrk_bf16(x.data_ptr(), 128, x.data_ptr(), 256, 256, 256, 1, 0, 0) == -2  # pitch < width
-    assert lib.muon_hip_syrk_bf16(None, 256, x.data_ptr(), 256, 256, 256, 1, 0, 0) == -1
-    assert lib.muon_hip_syrk_bf16(x.data_ptr(), 256, x.data_ptr(), 256, 256, 256, 1, 99, 0) == -1
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 128, 128, 1, abi.CFG_256_PIPE, 0) == -2  # 128 is not a 256-tile
+    assert lib.muon_hip_syrk_bf16(None, x.data_ptr(), 256, 256, 1, 0, 0) == -1
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 256, 256, 1, 99, 0) == -1
     with pytest.raises(abi.MuonHipError):
-        abi.check(lib.muon_hip_bx_axpy_bf16(x.data_ptr(), 256, x.data_ptr(), 256, None, 256, None, 256, 256, 1, 1.0, 0, 0))
+        abi.check(lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), None, None, 256, 256, 1, 1.0, 0, 0))
 
 
 NS_SHAPES = [(64, 160), (160, 64), (33, 47), (100, 300), (300, 100), (128, 896), (896, 128), (256, 256), (512, 1024)]

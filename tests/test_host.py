@@ -157,7 +157,7 @@ def test_host_only_entry_points():
     assert w1 >= 8 * 896 * 4864 + 4 * 896 * 896 and w1 < w2 <= 2 * w1 + 4096
     assert lib.muon_hip_workspace_bytes(0, 4, 1) == 0 and b"positive" in lib.muon_hip_last_error()
     assert lib.muon_hip_set_gemm_config(99) == -1
-    assert lib.muon_hip_set_gemm_config(_abi.CFG_256x256_W4) == 0
+    assert lib.muon_hip_set_gemm_config(_abi.CFG_256_PIPE) == 0
     try:
         assert _abi.geometry(896, 4864)["tile"] == 256 and _abi.geometry(896, 4864)["Mp"] == 1024
     finally:
