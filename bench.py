@@ -153,6 +153,9 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the workload's own)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--workspace-limit-gib", type=float, default=0.0,
+                    help="cap of the Newton-Schulz workspace (0 = the optimizer's default); smaller caps mean more, "
+                         "smaller grouped launches")
     ap.add_argument("--extras", action="store_true",
                     help="also time the two neighbours of the Muon step, outside the timed region: gradient-norm clipping "
                          "over the same gradients and the AdamW fallback over an embedding + lm_head + norm-vector group")
@@ -188,7 +191,8 @@ def main():
         params.append(torch.nn.Parameter((0.02 * torch.randn(*s, device=dev, generator=gen)).to(pd)))
     for p in params:
         p.grad = (1e-3 * torch.randn(*p.shape, device=dev, generator=gen)).to(pd)
-    opt = Muon([dict(params=list(params), use_muon=True, **HP)], momentum_dtype=md if pd != torch.float32 else None)
+    extra = dict(workspace_limit_bytes=int(args.workspace_limit_gib * (1 << 30))) if args.workspace_limit_gib > 0 else {}
+    opt = Muon([dict(params=list(params), use_muon=True, **HP)], momentum_dtype=md if pd != torch.float32 else None, **extra)
 
     flops_step = sum(ns_flops(*s, HP["ns_steps"]) for s in shapes)
     elements = sum(s[0] * s[1] for s in shapes)
