@@ -47,11 +47,17 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// Workgroups are dealt to the 8 XCDs round-robin by their linear id.  Give each XCD a
-// contiguous range of logical ids instead, so tiles that share operands share an L2.
+// Workgroups are dealt to the 8 XCDs round-robin by their linear id.  Give each XCD runs of
+// XCD_CHUNK consecutive logical ids instead (one round of its 32 CUs), so tiles that share operands
+// share an L2, and deal those runs to the XCDs in turn, so that at any time all eight work on
+// neighbouring tiles of the same matrix and the memory-side cache, which all XCDs share, serves
+// the panels the others have already fetched.
+#ifndef XCD_CHUNK
+#define XCD_CHUNK 32
+#endif
 __device__ __forceinline__ int xcd_remap(int pid, int nblocks) {
-    const int q = nblocks / XCD_COUNT, r = nblocks % XCD_COUNT;
+    const int full = nblocks / (XCD_COUNT * XCD_CHUNK) * (XCD_COUNT * XCD_CHUNK);
+    if (pid >= full) return pid;
     const int xcd = pid % XCD_COUNT, local = pid / XCD_COUNT;
-    const int base = xcd * q + (xcd < r ? xcd : r);
-    return base + local;
+    return ((local / XCD_CHUNK) * XCD_COUNT + xcd) * XCD_CHUNK + local % XCD_CHUNK;
 }
