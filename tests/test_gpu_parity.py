@@ -206,7 +206,7 @@ def test_newton_schulz_small_shapes(env, rows, cols):
 
 
 def test_newton_schulz_config1(env):
-    """BASELINE config 1: 896x4864 fp32 N(0,1) from seed 0, five bf16 iterations."""
+    """Benchmark config 1: 896x4864 fp32 N(0,1) from seed 0, five bf16 iterations."""
     print("ns config 1", flush=True)
     O, mu = env["O"], env["mu"]
     G = torch.randn(896, 4864, generator=torch.Generator().manual_seed(0))
@@ -318,7 +318,7 @@ def _check_step(opt, orc, gp, cp, grads, dtype, p_tol):
 
 
 def test_full_step_small_param_set_three_steps(env):
-    """A 2-layer slice of the Qwen2.5-0.5B-shaped set (BASELINE config 2 hyper-parameters),
+    """A 2-layer slice of the Qwen2.5-0.5B-shaped set (benchmark config 2 hyper-parameters),
     three consecutive steps, fp32 everything, plus a small AdamW-fallback group."""
     print("full step, 2 layers x 3 steps", flush=True)
     weights, grads = make_param_set(QWEN25_05B, layers=2, seed=1, steps=3)
@@ -482,7 +482,7 @@ def test_matmul_transpose_api(env):
 
 
 def test_config2_full_size_sampled_parity(env):
-    """BASELINE config 2 at full size (24 layers, 168 matrices, 3 steps) on the GPU; the
+    """Benchmark config 2 at full size (24 layers, 168 matrices, 3 steps) on the GPU; the
     oracle checks layer 0 and layer 23 (matrices are independent, so a sample is exact)."""
     print("config 2 full size", flush=True)
     mu, O = env["mu"], env["O"]
@@ -526,7 +526,7 @@ def _sv_band(out: torch.Tensor, probes: int = 8):
 
 @pytest.mark.parametrize("rows,cols", [(4096, 12288), (8192, 8192), (28672, 8192)])
 def test_full_size_newton_schulz(env, rows, cols):
-    """BASELINE config 3's largest shape and config 4's two matrices (N(0,1), seed 2, 5 iterations)
+    """Benchmark config 3's largest shape and config 4's two matrices (N(0,1), seed 2, 5 iterations)
     at full size: against the oracle on the host cores, and through properties that do not need it
     (transpose equivariance and power-of-two scale invariance are exact; singular values land in the band)."""
     print(f"full-size NS {rows}x{cols}", flush=True)
@@ -554,7 +554,7 @@ def test_full_size_newton_schulz(env, rows, cols):
 
 
 def test_config3_one_layer_full_step(env):
-    """BASELINE config 3 shapes (Qwen3-8B layer: bf16 params and grads, fp32 momentum), two layers so that
+    """Benchmark config 3 shapes (Qwen3-8B layer: bf16 params and grads, fp32 momentum), two layers so that
     every bucket is a grouped launch; the oracle steps every matrix of layer 0 for two steps."""
     print("config 3 layer", flush=True)
     from tests.helpers import QWEN3_8B
@@ -584,7 +584,7 @@ def test_config3_one_layer_full_step(env):
 
 
 def test_config5_moe_layer_sampled_parity(env):
-    """BASELINE config 5 shapes (Qwen3-MoE-30B-A3B: 128 experts x (gate, up 768x2048; down 2048x768) plus
+    """Benchmark config 5 shapes (Qwen3-MoE-30B-A3B: 128 experts x (gate, up 768x2048; down 2048x768) plus
     attention q 4096x2048, k, v 512x2048, o 2048x4096; grads N(0, 1e-3) seed 3, bf16 params, fp32 momentum):
     one full layer, 388 matrices in 5 grouped buckets; the oracle steps a sample out of every bucket."""
     print("config 5 layer", flush=True)
