@@ -31,7 +31,10 @@ struct GemmArgs {
     long strideEt;
     int cbEt;
     float s0, s1;           // SYMPOLY: (b, c); BX: (a, -)
+    int big_blocks;         // set by the launcher: workgroups that compute whole 256x256 tiles (split-tail kernel)
 };
+
+constexpr int GEMM_CU_COUNT = 256;  // compute units of the part: one 256x256 workgroup each
 
 int gemm_cfg_tile(int cfg);
 hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t stream);

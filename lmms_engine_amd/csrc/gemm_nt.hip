@@ -73,15 +73,20 @@ __device__ __forceinline__ const T* uniform_ptr(const T* p) {
     return (const T*)(((unsigned long long)hi << 32) | lo);
 }
 
+// Tile `logical` (0 .. tiles_per_mat * batch - 1) in the launch order: matrix by matrix, 4-row groups.
 template <int EPI>
-__device__ __forceinline__ TileCoord decode_tile(const GemmArgs& g) {
-    const int logical = xcd_remap(blockIdx.x, gridDim.x);
+__device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int logical) {
     TileCoord tc;
     tc.bidx = logical / g.tiles_per_mat;
     const int t = logical - tc.bidx * g.tiles_per_mat;
     if (EPI == EPI_BX) rect_decode<4>(t, g.tiles_m, g.tiles_n, tc.ti, tc.tj);
     else tri_decode<4>(t, g.tiles_m, tc.ti, tc.tj);
     return tc;
+}
+
+template <int EPI>
+__device__ __forceinline__ TileCoord decode_tile(const GemmArgs& g) {
+    return tile_of<EPI>(g, xcd_remap(blockIdx.x, gridDim.x));
 }
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
@@ -532,7 +537,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe4_kernel(const Gemm
 // loads of k-tile t+4 into it are issued in p=2t+2 / 2t+3, each wave waits for its own at the
 // end of its M phase two k-tiles later (p=2t+6 / 2t+7), and k-tile t+4 is first read in p=2t+8.
 template <int BM, int BN, int WGM, int WGN, int EPI>
-__global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArgs g) {
+__device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, unsigned char* smem) {
     constexpr int NW = WGM * WGN;
     constexpr int BK4 = 32, ROWB = 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -544,13 +549,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
     static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "dma split");
     static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
 
-    extern __shared__ __align__(16) unsigned char smem[];
-
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2;
     const int wm = wave / WGN, wn = wave % WGN;
-    const TileCoord tc = decode_tile<EPI>(g);
     const int kb = g.kdim / BLK_COLS;
     const bf16_t* Pb = uniform_ptr(g.P + tc.bidx * g.strideP + panel_offset(tc.ti * BM, kb));
     const bf16_t* Qb = uniform_ptr(g.Q + tc.bidx * g.strideQ + panel_offset(tc.tj * BN, kb));
@@ -671,6 +673,32 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
     epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 }
 
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArgs g) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    pp_tile<BM, BN, WGM, WGN, EPI>(g, decode_tile<EPI>(g), smem);
+}
+
+// The same with a split tail: when the tile count leaves the last round of the 256 CUs mostly empty,
+// the first g.big_blocks workgroups compute 256x256 tiles as above and every remaining tile is cut
+// into four 128x128 tiles, one workgroup each, which fill the CUs that would otherwise idle for a
+// whole tile time.  The lower-left quarter of a diagonal tile of the symmetric kernels is the mirror
+// of the upper-right one and is skipped.
+template <int EPI>
+__global__ void __launch_bounds__(512) gemm_nt_pp_tail_kernel(const GemmArgs g) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    if ((int)blockIdx.x < g.big_blocks) {
+        pp_tile<256, 256, 2, 4, EPI>(g, tile_of<EPI>(g, xcd_remap(blockIdx.x, g.big_blocks)), smem);
+    } else {
+        const int s = blockIdx.x - g.big_blocks, quarter = s & 3;
+        TileCoord tc = tile_of<EPI>(g, g.big_blocks + (s >> 2));
+        if (EPI != EPI_BX && tc.ti == tc.tj && quarter == 2) return;
+        tc.ti = tc.ti * 2 + (quarter >> 1);
+        tc.tj = tc.tj * 2 + (quarter & 1);
+        pp_tile<128, 128, 2, 4, EPI>(g, tc, smem);
+    }
+}
+
 template <int BM, int BN, int WGM, int WGN, int EPI, int FEED>
 hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
     constexpr int stages = 2 * (BM + BN) * ROW_BYTES, epi = epilogue_bytes<BM, BN>();
@@ -714,9 +742,36 @@ int gemm_cfg_tile(int cfg) {
     }
 }
 
+template <int EPI>
+hipError_t launch_pp_tail(GemmArgs g, int nblocks, int rest, hipStream_t stream) {
+    constexpr int stages = 2 * (256 + 256) * ROW_BYTES, epi = epilogue_bytes<256, 256>();
+    constexpr int smem = stages > epi ? stages : epi;  // the 128-tiles need less of both
+    static bool configured = false;
+    auto kern = gemm_nt_pp_tail_kernel<EPI>;
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return e;
+        configured = true;
+    }
+    g.big_blocks = nblocks - rest;
+    hipLaunchKernelGGL(kern, dim3(g.big_blocks + 4 * rest), dim3(512), smem, stream, g);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t stream) {
     const int nblocks = g.tiles_per_mat * g.batch;
     if (nblocks <= 0) return hipSuccess;
+    // Ping-pong kernel: split the tiles of a last round that would fill at most a quarter of the CUs (a 128x128
+    // tile takes about 0.6 of the time of a 256x256 one, so one round of quarters beats a round of whole tiles).
+    const int rest = nblocks % GEMM_CU_COUNT;
+    if (cfg == GEMM_CFG_256_PINGPONG && nblocks > GEMM_CU_COUNT && rest > 0 && rest <= GEMM_CU_COUNT / 4) {
+        switch (epi) {
+            case EPI_SYRK: return launch_pp_tail<EPI_SYRK>(g, nblocks, rest, stream);
+            case EPI_SYMPOLY: return launch_pp_tail<EPI_SYMPOLY>(g, nblocks, rest, stream);
+            case EPI_BX: return launch_pp_tail<EPI_BX>(g, nblocks, rest, stream);
+            default: return hipErrorInvalidValue;
+        }
+    }
     switch (epi) {
         case EPI_SYRK: return launch_cfg<EPI_SYRK>(cfg, g, nblocks, stream);
         case EPI_SYMPOLY: return launch_cfg<EPI_SYMPOLY>(cfg, g, nblocks, stream);

@@ -177,6 +177,37 @@ def test_bx_axpy_rounding_points(env, cfg, outputs):
         assert torch.equal(Xo, XTo.mT)
 
 
+def test_split_tail_is_bitwise_the_plain_kernel(env):
+    """A tile count just above a multiple of the 256 CUs makes the ping-pong configuration cut the last tiles into
+    128x128 quarters.  Every output element still sums its products in ascending k, so the result equals the
+    two-stage 256-tile kernel's bit for bit (which never splits)."""
+    lib, abi, dev, O = env["lib"], env["abi"], env["dev"], env["O"]
+    g = torch.Generator().manual_seed(77)
+    # X.Xt: 10 triangular tiles x 26 matrices = 260; b.A + c.A.A likewise; a.X + B.X: 4 x 2 tiles x 33 = 264
+    M, K, batch = 1024, 256, 26
+    Xb = _pack(env, (torch.randn(batch, M, K, generator=g) / 16).bfloat16().to(dev))
+    outs = []
+    for cfg in (abi.CFG_256_PINGPONG, abi.CFG_256_PIPE):
+        Ab, Bb = _blocked_nan(env, batch, M, M), _blocked_nan(env, batch, M, M)
+        abi.check(lib.muon_hip_syrk_bf16(Xb.data_ptr(), Ab.data_ptr(), M, K, batch, cfg, 0))
+        abi.check(lib.muon_hip_sympoly_bf16(Ab.data_ptr(), Bb.data_ptr(), M, batch, O.NS_COEFFS[1], O.NS_COEFFS[2], cfg, 0))
+        outs.append((_unpack(env, Ab, batch, M, M), _unpack(env, Bb, batch, M, M)))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert torch.equal(outs[0][0], outs[0][0].mT) and not torch.isnan(outs[0][1]).any()
+    M, K, batch = 1024, 512, 33
+    XT = _pack(env, (torch.randn(batch, K, M, generator=g) / 16).bfloat16().to(dev))
+    Bm = (torch.randn(batch, M, M, generator=g) / 16).bfloat16()
+    Bb = _pack(env, (torch.triu(Bm) + torch.triu(Bm, 1).mT).to(dev))
+    outs = []
+    for cfg in (abi.CFG_256_PINGPONG, abi.CFG_256_PIPE):
+        Xo, XTo = _blocked_nan(env, batch, M, K), _blocked_nan(env, batch, K, M)
+        abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), XT.data_ptr(), Xo.data_ptr(), XTo.data_ptr(), M, K, batch,
+                                            O.NS_COEFFS[0], cfg, 0))
+        outs.append((_unpack(env, Xo, batch, M, K), _unpack(env, XTo, batch, K, M)))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    assert torch.equal(outs[0][0], outs[0][1].mT) and not torch.isnan(outs[0][0]).any()
+
+
 def test_gemm_entry_points_reject_bad_shapes(env):
     lib, abi = env["lib"], env["abi"]
     x = torch.zeros(256 * 256, dtype=torch.bfloat16, device=env["dev"])
