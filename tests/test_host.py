@@ -164,3 +164,30 @@ def test_host_only_entry_points():
         assert lib.muon_hip_set_gemm_config(_abi.CFG_AUTO) == 0
     with pytest.raises(TypeError):
         _abi.dtype_code(torch.float16)
+
+
+def test_clip_grad_norm_host_behaviour():
+    """What clip_grad_norm_ decides before any kernel runs: the empty cases return what torch's
+    _get_total_norm returns, other norms and CPU gradients are refused (no fallback path)."""
+    from lmms_engine_amd import _abi, clip_grad
+
+    out = clip_grad.clip_grad_norm_([], 1.0)
+    assert out.item() == 0.0 and out.device.type == "cpu"
+    p = torch.nn.Parameter(torch.zeros(4))
+    assert clip_grad.clip_grad_norm_(p, 1.0).item() == 0.0  # a bare tensor is accepted; no grad yet
+    p.grad = torch.ones(4)
+    with pytest.raises(NotImplementedError):
+        clip_grad.clip_grad_norm_([p], 1.0, norm_type=float("inf"))
+    with pytest.raises(_abi.MuonHipError):
+        clip_grad.clip_grad_norm_([p], 1.0)
+    assert torch.equal(p.grad, torch.ones(4))  # untouched
+    assert clip_grad.fsdp2_clip_grad_norm_ is clip_grad.clip_grad_norm_
+
+
+def test_tensor_list_table_rejects_cpu_tensors():
+    from lmms_engine_amd import _abi
+    from lmms_engine_amd.multi_tensor import TensorListTable
+
+    with pytest.raises(_abi.MuonHipError):
+        TensorListTable([[torch.zeros(3)]])
+    assert _abi.MULTI_CHUNK == 16384
