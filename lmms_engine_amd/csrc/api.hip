@@ -89,7 +89,8 @@ bool use_tile256(int M) { return M % 256 == 0 && M >= 512; }
 // kernel wherever 256-tiles fill the machine, 128-tiles for the symmetric products of small matrices.
 int pick_cfg(int M, int epi = EPI_BX, int kdim = 0) {
     if (g_forced_cfg != MUON_HIP_CFG_AUTO) return g_forced_cfg;
-    if (!use_tile256(M)) return (epi == EPI_SYRK && kdim < 2048) ? GEMM_CFG_128_PIPE4 : GEMM_CFG_128_PIPE;
+    (void)kdim;
+    if (!use_tile256(M)) return GEMM_CFG_128_PIPE;
     if (epi != EPI_BX && M <= 512) return GEMM_CFG_128_PIPE;
     return GEMM_CFG_256_PINGPONG;
 }
