@@ -55,10 +55,8 @@ extern "C" {
 #define MUON_HIP_CFG_AUTO (-1)
 #define MUON_HIP_CFG_128_PIPE 0      /* 128x128 tile, 4 waves, 64-column k-tiles, two LDS stages */
 #define MUON_HIP_CFG_256_PIPE 1      /* 256x256 tile, 8 waves, the same pipeline */
-#define MUON_HIP_CFG_128_PIPE4 2     /* 128x128 tile, 4 waves, 32-column k-tiles, four LDS stages */
-#define MUON_HIP_CFG_256_W4_PIPE4 3  /* 256x256 tile, 4 waves of 128x128, four LDS stages */
-#define MUON_HIP_CFG_256_PINGPONG 4  /* 256x256 tile, two groups of 4 waves alternating memory / MFMA phases */
-#define MUON_HIP_CFG_COUNT 5
+#define MUON_HIP_CFG_256_PINGPONG 2  /* 256x256 tile, two groups of 4 waves alternating memory / MFMA phases */
+#define MUON_HIP_CFG_COUNT 3
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);
@@ -141,10 +139,11 @@ int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cf
 /* B = bf16(bf16(b*A) + bf16(c*bf16(A A))) for symmetric A (Mp x Mp): muon_utils.py:150-151. */
 int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* stream);
 
-/* X' = bf16(bf16(a*X) + bf16(B X)): muon_utils.py:152.  B (Mp x Mp) symmetric, XT (Kp x Mp) the
- * transposed copy of X; writes Xout (Mp x Kp) and/or XTout (Kp x Mp) (either may be null, not both). */
-int muon_hip_bx_axpy_bf16(const void* B, const void* XT, void* Xout, void* XTout, int Mp, int Kp, int batch, double a,
-                          int cfg, void* stream);
+/* X' = bf16(bf16(a*X) + bf16(B X)): muon_utils.py:152.  B (Mp x Mp) symmetric, X and Xout (Mp x Kp) distinct
+ * buffers.  The reduction runs down the columns of X, which the kernel reads from LDS with gfx950's
+ * transposing read, so no transposed copy of X exists anywhere. */
+int muon_hip_bx_axpy_bf16(const void* B, const void* X, void* Xout, int Mp, int Kp, int batch, double a, int cfg,
+                          void* stream);
 
 /* ---- AdamW fallback ------------------------------------------------------------------ */
 

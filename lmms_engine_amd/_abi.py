@@ -15,8 +15,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmuon_hip.so")
 
 F32, BF16 = 0, 1
-CFG_AUTO, CFG_128_PIPE, CFG_256_PIPE, CFG_128_PIPE4, CFG_256_W4_PIPE4, CFG_256_PINGPONG = -1, 0, 1, 2, 3, 4
-GEMM_CONFIGS = list(range(5))
+CFG_AUTO, CFG_128_PIPE, CFG_256_PIPE, CFG_256_PINGPONG = -1, 0, 1, 2
+GEMM_CONFIGS = list(range(3))
 K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW, K_ADAMW_MULTI, K_GRAD_NORM, K_CLIP_SCALE = range(10)
 KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw", "adamw_multi",
                 "grad_norm", "clip_scale"]
@@ -44,8 +44,7 @@ SIGNATURES = {
     "muon_hip_unpack_bf16": (c_int, [c_void_p, c_int, c_int, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p]),
     "muon_hip_syrk_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "muon_hip_sympoly_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_double, c_double, c_int, c_void_p]),
-    "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_int,
-                                      c_void_p]),
+    "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_int, c_void_p]),
     "muon_hip_adamw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_double,
                                c_double, c_double, c_double, c_void_p]),
     "muon_hip_adamw_multi": (c_int, [c_void_p] * 8 + [c_int, c_long, c_int] + [c_double] * 5 + [c_void_p]),

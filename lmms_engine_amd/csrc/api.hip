@@ -76,8 +76,8 @@ struct Timed {
 struct Plan {
     int rows, cols, batch, M, K, Mp, Kp, tile, cfg, nparts;
     bool transposed;
-    long n, strideU, strideX, strideXT, strideA;  // elements per matrix: U dense, the others blocked
-    size_t offX[2], offXT[2], offA, offB, offParts, offDenom, total;
+    long n, strideU, strideX, strideA;  // elements per matrix: U dense, the others blocked
+    size_t offX[2], offA, offB, offParts, offDenom, total;
 };
 
 inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
@@ -112,7 +112,6 @@ int make_plan(int rows, int cols, int batch, Plan& p) {
     p.n = (long)rows * cols;
     p.strideU = round_up(p.n, 8);
     p.strideX = blocked_elems(p.Mp, p.Kp);
-    p.strideXT = blocked_elems(p.Kp, p.Mp);
     p.strideA = blocked_elems(p.Mp, p.Mp);
     p.nparts = momentum_parts(p.n);
     const long T = p.Mp / p.tile, TN = p.Kp / p.tile;
@@ -123,12 +122,10 @@ int make_plan(int rows, int cols, int batch, Plan& p) {
         off += (size_t)round_up((long)bytes, 256);
         return o;
     };
-    const size_t xb = (size_t)batch * p.strideX * 2, xtb = (size_t)batch * p.strideXT * 2;
+    const size_t xb = (size_t)batch * p.strideX * 2;
     const size_t ab = (size_t)batch * p.strideA * 2;
     p.offX[0] = seg(xb);
     p.offX[1] = seg(xb);  // doubles as U (the blend in the parameter's layout) before the first iteration
-    p.offXT[0] = seg(xtb);
-    p.offXT[1] = seg(xtb);
     p.offA = seg(ab);
     p.offB = seg(ab);
     p.offParts = seg((size_t)batch * p.nparts * sizeof(float));
@@ -195,14 +192,14 @@ int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b,
     return e == hipSuccess ? 0 : hip_fail(e, "sympoly launch");
 }
 
-int do_bx(int cfg, const bf16_t* B, const bf16_t* XT, bf16_t* Xout, bf16_t* XTout, int Mp, int Kp, int batch, double a,
-          hipStream_t s) {
+int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int Kp, int batch, double a, hipStream_t s) {
     GemmArgs g = {};
     const int tile = gemm_cfg_tile(cfg);
     g.P = B;
     g.strideP = blocked_elems(Mp, Mp);
-    g.Q = XT;
-    g.strideQ = blocked_elems(Kp, Mp);
+    g.Q = X;
+    g.strideQ = blocked_elems(Mp, Kp);
+    g.cbQ = Kp / BLK_COLS;
     g.kdim = Mp;
     g.tiles_m = Mp / tile;
     g.tiles_n = Kp / tile;
@@ -211,12 +208,9 @@ int do_bx(int cfg, const bf16_t* B, const bf16_t* XT, bf16_t* Xout, bf16_t* XTou
     g.C = Xout;
     g.strideC = blocked_elems(Mp, Kp);
     g.cbC = Kp / BLK_COLS;
-    g.Ct = XTout;
-    g.strideCt = blocked_elems(Kp, Mp);
-    g.cbCt = Mp / BLK_COLS;
-    g.Et = XT;
-    g.strideEt = blocked_elems(Kp, Mp);
-    g.cbEt = Mp / BLK_COLS;
+    g.Et = X;
+    g.strideEt = blocked_elems(Mp, Kp);
+    g.cbEt = Kp / BLK_COLS;
     g.s0 = (float)a;
     Timed t(MUON_HIP_K_BX, s);
     hipError_t e = launch_gemm_nt(cfg, EPI_BX, g, s);
@@ -294,24 +288,20 @@ int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int step
     if (steps < 0) return fail(MUON_HIP_EINVAL, "steps must be >= 0");
     hipStream_t s = (hipStream_t)stream;
     bf16_t* X[2] = {wsp(workspace, p.offX[0]), wsp(workspace, p.offX[1])};
-    bf16_t* XT[2] = {wsp(workspace, p.offXT[0]), wsp(workspace, p.offXT[1])};
     bf16_t* A = wsp(workspace, p.offA);
     bf16_t* B = wsp(workspace, p.offB);
     {
         Timed t(MUON_HIP_K_NORMALIZE, s);
         hipError_t e = launch_normalize(X[1], p.strideU, (const float*)((char*)workspace + p.offParts), p.nparts,
-                                        (float*)((char*)workspace + p.offDenom), X[0], p.strideX, XT[0], p.strideXT, rows,
-                                        cols, p.Mp, p.Kp, batch, s);
+                                        (float*)((char*)workspace + p.offDenom), X[0], p.strideX, rows, cols, p.Mp, p.Kp,
+                                        batch, s);
         if (e != hipSuccess) return hip_fail(e, "normalize launch");
     }
     int cur = 0;
     for (int it = 0; it < steps; ++it) {
-        const bool last = it + 1 == steps;
         if (int rc = do_syrk(pick_cfg(p.M, EPI_SYRK, p.Kp), X[cur], A, p.Mp, p.Kp, batch, s)) return rc;
         if (int rc = do_sympoly(pick_cfg(p.M, EPI_SYMPOLY), A, B, p.Mp, batch, b, c, s)) return rc;
-        bf16_t* xo = (last && p.transposed) ? nullptr : X[cur ^ 1];
-        bf16_t* xto = (last && !p.transposed) ? nullptr : XT[cur ^ 1];
-        if (int rc = do_bx(pick_cfg(p.M, EPI_BX), B, XT[cur], xo, xto, p.Mp, p.Kp, batch, a, s)) return rc;
+        if (int rc = do_bx(pick_cfg(p.M, EPI_BX), B, X[cur], X[cur ^ 1], p.Mp, p.Kp, batch, a, s)) return rc;
         cur ^= 1;
     }
     return 0;
@@ -324,12 +314,10 @@ int muon_hip_apply_update(const void* const* p_ptrs, int p_dtype, void* workspac
     if (int rc = check_ws(workspace)) return rc;
     if (!p_ptrs || !dtype_ok(p_dtype) || steps < 0) return fail(MUON_HIP_EINVAL, "bad pointer table, dtype or steps");
     hipStream_t s = (hipStream_t)stream;
-    const int cur = steps & 1;
-    const bf16_t* O = wsp(workspace, p.transposed ? p.offXT[cur] : p.offX[cur]);
-    const int cbo = (p.transposed ? p.Mp : p.Kp) / BLK_COLS;  // O is rows x cols in the parameter's orientation
-    const long strideO = p.transposed ? p.strideXT : p.strideX;
+    const bf16_t* O = wsp(workspace, p.offX[steps & 1]);  // X (M x K): the parameter's image, or its transpose when rows > cols
     Timed t(MUON_HIP_K_UPDATE, s);
-    hipError_t e = launch_apply_update(p_ptrs, p_dtype, O, strideO, cbo, rows, cols, batch, scale, lr, weight_decay, s);
+    hipError_t e = launch_apply_update(p_ptrs, p_dtype, O, p.strideX, p.Kp / BLK_COLS, rows, cols, batch, scale, lr,
+                                       weight_decay, s);
     return e == hipSuccess ? 0 : hip_fail(e, "apply_update launch");
 }
 
@@ -339,11 +327,8 @@ int muon_hip_ns_output(void* workspace, int rows, int cols, int batch, int steps
     if (int rc = check_ws(workspace)) return rc;
     if (!out || steps < 0) return fail(MUON_HIP_EINVAL, "bad output pointer or steps");
     hipStream_t s = (hipStream_t)stream;
-    const int cur = steps & 1;
-    const bf16_t* O = wsp(workspace, p.transposed ? p.offXT[cur] : p.offX[cur]);
-    const int cbo = (p.transposed ? p.Mp : p.Kp) / BLK_COLS;
-    const long strideO = p.transposed ? p.strideXT : p.strideX;
-    hipError_t e = launch_unpack((bf16_t*)out, p.n, cols, O, strideO, cbo, rows, cols, batch, s);
+    const bf16_t* O = wsp(workspace, p.offX[steps & 1]);
+    hipError_t e = launch_unpack((bf16_t*)out, p.n, cols, O, p.strideX, p.Kp / BLK_COLS, rows, cols, p.transposed, batch, s);
     return e == hipSuccess ? 0 : hip_fail(e, "ns_output launch");
 }
 
@@ -383,7 +368,7 @@ int muon_hip_unpack_bf16(const void* src, int rows_p, int cols_p, void* dst, lon
     if (rows <= 0 || cols <= 0 || rows > rows_p || cols > cols_p || ld < cols || cols_p % BLK_COLS || batch > 65535)
         return fail(MUON_HIP_ESHAPE, "unpack: need 0 < rows <= rows_p, 0 < cols <= cols_p, ld >= cols, cols_p %% 32 == 0");
     hipError_t e = launch_unpack((bf16_t*)dst, dst_stride, ld, (const bf16_t*)src, blocked_elems(rows_p, cols_p),
-                                 cols_p / BLK_COLS, rows, cols, batch, (hipStream_t)stream);
+                                 cols_p / BLK_COLS, rows, cols, false, batch, (hipStream_t)stream);
     return e == hipSuccess ? 0 : hip_fail(e, "unpack launch");
 }
 
@@ -403,15 +388,14 @@ int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, d
     return do_sympoly(cfg, (const bf16_t*)A, (bf16_t*)B, Mp, batch, b, c, (hipStream_t)stream);
 }
 
-int muon_hip_bx_axpy_bf16(const void* B, const void* XT, void* Xout, void* XTout, int Mp, int Kp, int batch, double a,
-                          int cfg, void* stream) {
+int muon_hip_bx_axpy_bf16(const void* B, const void* X, void* Xout, int Mp, int Kp, int batch, double a, int cfg,
+                          void* stream) {
     if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp, EPI_BX);
     int tile;
     if (int rc = check_gemm(cfg, Mp, Kp, batch, tile)) return rc;
-    if (!B || !XT || (!Xout && !XTout)) return fail(MUON_HIP_EINVAL, "null operand");
-    if (XTout == XT) return fail(MUON_HIP_EINVAL, "XTout must not alias XT");
-    return do_bx(cfg, (const bf16_t*)B, (const bf16_t*)XT, (bf16_t*)Xout, (bf16_t*)XTout, Mp, Kp, batch, a,
-                 (hipStream_t)stream);
+    if (!B || !X || !Xout) return fail(MUON_HIP_EINVAL, "null operand");
+    if (Xout == X) return fail(MUON_HIP_EINVAL, "Xout must not alias X");
+    return do_bx(cfg, (const bf16_t*)B, (const bf16_t*)X, (bf16_t*)Xout, Mp, Kp, batch, a, (hipStream_t)stream);
 }
 
 int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int dtype, long n, int step, double lr,

@@ -12,13 +12,12 @@ hipError_t launch_momentum_norm(const void* const* g_ptrs, const void* const* m_
 hipError_t launch_cast_norm(const void* G, long strideG, int g_dtype, bf16_t* U, long strideU, float* partials,
                             int nparts, long n, int batch, hipStream_t stream);
 hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, float* denom, bf16_t* X,
-                            long strideX, bf16_t* XT, long strideXT, int rows, int cols, int Mp, int Kp, int batch,
-                            hipStream_t stream);
+                            long strideX, int rows, int cols, int Mp, int Kp, int batch, hipStream_t stream);
 hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf16_t* O, long strideO, int cbo,
                                int rows, int cols, int batch, double scale, double lr, double wd,
                                hipStream_t stream);
 hipError_t launch_unpack(bf16_t* out, long strideOut, int ld, const bf16_t* O, long strideO, int cbo, int rows,
-                         int cols, int batch, hipStream_t stream);
+                         int cols, bool transposed, int batch, hipStream_t stream);
 hipError_t launch_pack(const bf16_t* src, long strideSrc, int ld, int rows, int cols, bf16_t* dst, long strideDst,
                        int rows_p, int cols_p, int batch, hipStream_t stream);
 hipError_t launch_adamw(void* p, const void* g, void* e1, void* e2, int dtype, long n, int step, double lr,

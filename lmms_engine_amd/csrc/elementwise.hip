@@ -1,5 +1,5 @@
 // HBM-bound kernels of the Muon step on gfx950: momentum/Nesterov blend with Frobenius
-// partial sums, normalisation into the two padded operand layouts, the scaled parameter
+// partial sums, normalisation into the blocked operand X, the scaled parameter
 // update, and the AdamW fallback.  128-bit accesses on the aligned path, a scalar path
 // otherwise.  All reductions are two-stage with a fixed order, so results are
 // run-to-run bit identical (no float atomics).
@@ -187,24 +187,22 @@ __global__ void __launch_bounds__(256) frob_finalize_kernel(const float* partial
     }
 }
 
-// One 64x128 tile of the bf16 blend u (parameter layout, rows x cols) divided by d, written
-// into the blocked operand that has u's orientation and, through an LDS transpose, into the other
-// one; both leave as 128-byte row pieces that are neighbours inside a 256x64 block (2 KB and 4 KB
-// contiguous per pass).  X is M x K, Xt is K x M, both zero padded to Mp x Kp / Kp x Mp.
+// One 64x128 tile of the bf16 blend u (parameter layout, rows x cols) divided by d, written into the
+// blocked X (M x K, zero padded to Mp x Kp): directly when the parameter has X's orientation
+// (16 rows of a block back to back = 1 KB runs), through an LDS transpose when rows > cols (X = u^T,
+// 32 rows of a block = 2 KB runs).
 __global__ void __launch_bounds__(256)
-normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, long strideX, bf16_t* XT,
-                 long strideXT, int rows, int cols, int Mp, int Kp) {
+normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, long strideX, int rows, int cols,
+                 int Mp, int Kp) {
     constexpr int TR = 64, TC = 128, PITCH = TC + 8;
     __shared__ __align__(16) bf16_t tile[TR][PITCH];
     const int b = blockIdx.y;
     const float d = denom[b];
     const bf16_t* u = U + b * strideU;
-    // transposed (rows > cols): X = u^T, so the padded image of u is Xt.
+    bf16_t* x = X + b * strideX;
     const bool transposed = rows > cols;
-    const int Cp = transposed ? Mp : Kp, Rp = transposed ? Kp : Mp;       // padded cols / rows of u's image
-    bf16_t* same = transposed ? XT + b * strideXT : X + b * strideX;      // same orientation as u
-    bf16_t* flip = transposed ? X + b * strideX : XT + b * strideXT;      // the transposed image
-    const int cb_same = Cp / BLK_COLS, cb_flip = Rp / BLK_COLS;
+    const int Cp = transposed ? Mp : Kp;  // padded columns of u's image
+    const int cbx = Kp / BLK_COLS;
     const int tiles_c = Cp / TC;
     const int r0 = (blockIdx.x / tiles_c) * TR, c0 = (blockIdx.x % tiles_c) * TC;
     const int tr = threadIdx.x >> 4, tc = (threadIdx.x & 15) * 8;  // 16 rows x 16 chunks per pass
@@ -226,11 +224,12 @@ normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, l
         bf16x8 o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[i] = f2bf(__fdiv_rn(bf2f(v[h][i]), d));
-        *(bf16x8*)(&tile[tr + h * 16][tc]) = o;
-        *(bf16x8*)(same + blocked_offset(r, c, cb_same)) = o;
+        if (transposed) *(bf16x8*)(&tile[tr + h * 16][tc]) = o;
+        else *(bf16x8*)(x + blocked_offset(r, c, cbx)) = o;
     }
+    if (!transposed) return;
     __syncthreads();
-    // flip[c][r]: 128 rows of 64 elements; a thread gathers 8 consecutive r of one column
+    // X[c][r]: 128 rows of 64 elements; a thread gathers 8 consecutive r of one column of the tile
     const int fr = (threadIdx.x & 7) * 8, fc0 = threadIdx.x >> 3;  // 8 chunks per row, 32 rows per pass
 #pragma unroll
     for (int h = 0; h < 4; ++h) {
@@ -238,7 +237,7 @@ normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, l
         bf16x8 o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[i] = tile[fr + i][fc];
-        *(bf16x8*)(flip + blocked_offset(c0 + fc, r0 + fr, cb_flip)) = o;
+        *(bf16x8*)(x + blocked_offset(c0 + fc, r0 + fr, cbx)) = o;
     }
 }
 
@@ -304,16 +303,59 @@ apply_update_kernel(const void* const* p_ptrs, const bf16_t* O, long strideO, in
     }
 }
 
-// A blocked matrix into a dense row-major bf16 tensor (row pitch ld): the NS output of
+// The same for a parameter with rows > cols, whose update is X^T: one tile of 64 parameter rows x 128 parameter
+// columns is read from X as 128 rows of 64 elements (8 KB runs of two blocks), transposed through LDS and applied
+// to 256-byte (bf16) or 512-byte (fp32) pieces of the parameter's rows.
+template <typename PT>
+__global__ void __launch_bounds__(256)
+apply_update_t_kernel(const void* const* p_ptrs, const bf16_t* O, long strideO, int cbo, int rows, int cols,
+                      UpdateMath um) {
+    constexpr int TR = 64, TC = 128, PITCH = TR + 8;
+    __shared__ __align__(16) bf16_t tile[TC][PITCH];  // tile[c][r]
+    const int b = blockIdx.y;
+    PT* p = (PT*)p_ptrs[b];
+    const bf16_t* o = O + b * strideO;
+    const int tiles_c = (cols + TC - 1) / TC;
+    const int r0 = (blockIdx.x / tiles_c) * TR, c0 = (blockIdx.x % tiles_c) * TC;
+    // X rows c0..c0+127, columns r0..r0+63 (always inside the padded X): 8 chunks per row, 32 rows per pass
+    const int xr = threadIdx.x >> 3, xc = (threadIdx.x & 7) * 8;
+#pragma unroll
+    for (int h = 0; h < 4; ++h)
+        *(bf16x8*)(&tile[xr + h * 32][xc]) = *(const bf16x8*)(o + blocked_offset(c0 + xr + h * 32, r0 + xc, cbo));
+    __syncthreads();
+    const bool vec = (cols % 8 == 0) && ((((uintptr_t)p) & 15) == 0);
+    const int pr = threadIdx.x >> 4, pc = (threadIdx.x & 15) * 8;  // 16 rows x 16 chunks per pass
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+        const int r = r0 + pr + h * 16, c = c0 + pc;
+        if (r >= rows || c >= cols) continue;
+        float ov[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ov[i] = bf2f(tile[pc + i][pr + h * 16]);
+        PT* dst = p + (long)r * cols + c;
+        if (vec) {
+            float pv[8];
+            Ld<PT>::template load8<true>(dst, pv);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pv[i] = update_one<PT>(pv[i], ov[i], um);
+            Ld<PT>::template store8<true>(dst, pv);
+        } else {
+            for (int i = 0; i < 8 && c + i < cols; ++i) Ld<PT>::store(dst + i, update_one<PT>(Ld<PT>::load(dst + i), ov[i], um));
+        }
+    }
+}
+
+// A blocked matrix, or its transpose, into a dense row-major bf16 tensor (row pitch ld): the NS output of
 // fast_newtonschulz called alone, and the result of a single GEMM.
 __global__ void __launch_bounds__(256)
-unpack_kernel(bf16_t* out, long strideOut, int ld, const bf16_t* O, long strideO, int cbo, int rows, int cols) {
+unpack_kernel(bf16_t* out, long strideOut, int ld, const bf16_t* O, long strideO, int cbo, int rows, int cols,
+              int transposed) {
     const int b = blockIdx.y;
     const long n = (long)rows * cols;
     for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
         const long r = i / cols;
         const int c = (int)(i - r * cols);
-        out[b * strideOut + r * ld + c] = O[b * strideO + blocked_offset(r, c, cbo)];
+        out[b * strideOut + r * ld + c] = O[b * strideO + (transposed ? blocked_offset(c, r, cbo) : blocked_offset(r, c, cbo))];
     }
 }
 
@@ -413,16 +455,16 @@ hipError_t launch_cast_norm(const void* G, long strideG, int g_dtype, bf16_t* U,
 }
 
 hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, float* denom, bf16_t* X,
-                            long strideX, bf16_t* XT, long strideXT, int rows, int cols, int Mp, int Kp, int batch,
-                            hipStream_t stream) {
+                            long strideX, int rows, int cols, int Mp, int Kp, int batch, hipStream_t stream) {
     hipLaunchKernelGGL(frob_finalize_kernel, dim3(batch), dim3(256), 0, stream, partials, nparts, denom);
     // u's padded image is Rp x Cp with Rp a multiple of 64 and Cp a multiple of 128 (both are multiples of the tile edge)
     dim3 grid((Mp / 64) * (Kp / 64) / 2, batch), block(256);
-    hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, strideX, XT, strideXT, rows, cols,
-                       Mp, Kp);
+    hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, strideX, rows, cols, Mp, Kp);
     return hipGetLastError();
 }
 
+// O is X (M x K, blocked with cbo column blocks): the update in the parameter's orientation when rows <= cols,
+// its transpose otherwise.
 hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf16_t* O, long strideO, int cbo,
                                int rows, int cols, int batch, double scale, double lr, double wd,
                                hipStream_t stream) {
@@ -430,7 +472,18 @@ hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf1
     um.scale = (float)scale;
     um.decay = (float)(1.0 - lr * wd);
     um.alpha = (float)(-lr);
-    dim3 grid(blocks_for((long)rows * cols, 16384, 8192), batch), block(256);
+    dim3 block(256);
+    if (rows > cols) {
+        dim3 grid(((rows + 63) / 64) * ((cols + 127) / 128), batch);
+        if (p_dtype == MUON_HIP_F32)
+            hipLaunchKernelGGL((apply_update_t_kernel<float>), grid, block, 0, stream, p_ptrs, O, strideO, cbo, rows, cols, um);
+        else if (p_dtype == MUON_HIP_BF16)
+            hipLaunchKernelGGL((apply_update_t_kernel<bf16_t>), grid, block, 0, stream, p_ptrs, O, strideO, cbo, rows, cols, um);
+        else
+            return hipErrorInvalidValue;
+        return hipGetLastError();
+    }
+    dim3 grid(blocks_for((long)rows * cols, 16384, 8192), batch);
     if (p_dtype == MUON_HIP_F32)
         hipLaunchKernelGGL((apply_update_kernel<float>), grid, block, 0, stream, p_ptrs, O, strideO, cbo, rows, cols, um);
     else if (p_dtype == MUON_HIP_BF16)
@@ -442,9 +495,10 @@ hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf1
 }
 
 hipError_t launch_unpack(bf16_t* out, long strideOut, int ld, const bf16_t* O, long strideO, int cbo, int rows,
-                         int cols, int batch, hipStream_t stream) {
+                         int cols, bool transposed, int batch, hipStream_t stream) {
     dim3 grid(blocks_for((long)rows * cols, 256 * 8, 2048), batch), block(256);
-    hipLaunchKernelGGL(unpack_kernel, grid, block, 0, stream, out, strideOut, ld, O, strideO, cbo, rows, cols);
+    hipLaunchKernelGGL(unpack_kernel, grid, block, 0, stream, out, strideOut, ld, O, strideO, cbo, rows, cols,
+                       transposed ? 1 : 0);
     return hipGetLastError();
 }
 

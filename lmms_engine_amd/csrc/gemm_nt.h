@@ -5,29 +5,28 @@
 
 enum { EPI_SYRK = 0, EPI_SYMPOLY = 1, EPI_BX = 2 };
 enum {
-    GEMM_CFG_128_PIPE = 0,       // 128x128 tile, 4 waves, 64-column k-tiles in two LDS stages
-    GEMM_CFG_256_PIPE = 1,       // 256x256 tile, 8 waves, the same pipeline
-    GEMM_CFG_128_PIPE4 = 2,      // 128x128 tile, 4 waves, 32-column k-tiles in four LDS stages
-    GEMM_CFG_256_W4_PIPE4 = 3,   // 256x256 tile, 4 waves (128x128 each), four stages
-    GEMM_CFG_256_PINGPONG = 4,   // 256x256 tile, 8 waves in two alternating groups, four stages
-    GEMM_CFG_COUNT = 5
+    GEMM_CFG_128_PIPE = 0,      // 128x128 tile, 4 waves, 64-column k-tiles in two LDS stages
+    GEMM_CFG_256_PIPE = 1,      // 256x256 tile, 8 waves, the same pipeline
+    GEMM_CFG_256_PINGPONG = 2,  // 256x256 tile, 8 waves in two alternating groups, four stages of 32 columns
+    GEMM_CFG_COUNT = 3
 };
 
 struct GemmArgs {
     const bf16_t* P;        // left operand: rows x kdim, blocked
-    const bf16_t* Q;        // right operand: rows x kdim, blocked
+    const bf16_t* Q;        // right operand, blocked: rows x kdim (SYRK, SYMPOLY) or kdim x columns (BX)
     long strideP, strideQ;  // elements between matrices of the batch
+    int cbQ;                // BX: column blocks of Q
     int kdim;               // reduction length, a multiple of 128
     int tiles_m, tiles_n;   // tile grid of one matrix (triangular kernels: tiles_m == tiles_n)
     int tiles_per_mat;      // tiles_m*(tiles_m+1)/2 for the symmetric kernels, tiles_m*tiles_n for BX
     int batch;
-    bf16_t* C;              // out[i][j], blocked with cbC column blocks; may be null for BX
+    bf16_t* C;              // out[i][j], blocked with cbC column blocks
     long strideC;
     int cbC;
-    bf16_t* Ct;             // out[j][i], blocked; the same buffer as C for the symmetric kernels; may be null for BX
+    bf16_t* Ct;             // symmetric kernels: out[j][i], the same buffer as C; BX: unused
     long strideCt;
     int cbCt;
-    const bf16_t* Et;       // elementwise source read as Et[j][i], blocked: A (symmetric) or Xt
+    const bf16_t* Et;       // elementwise source, blocked: A read as Et[j][i] (symmetric), or X read as Et[i][j] (BX)
     long strideEt;
     int cbEt;
     float s0, s1;           // SYMPOLY: (b, c); BX: (a, -)

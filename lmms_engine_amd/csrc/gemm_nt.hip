@@ -1,18 +1,18 @@
-// NT GEMM family for the Newton-Schulz chain on gfx950 (v_mfma_f32_32x32x16_bf16).
+// GEMM family for the Newton-Schulz chain on gfx950 (v_mfma_f32_32x32x16_bf16).
 //
-// All three products of one NS iteration are "row times row" contractions of bf16
-// operands whose reduction dimension is contiguous:
-//   SYRK     A  = bf(X Xt)                         P = Q = X   (M x K)
-//   SYMPOLY  B  = bf(bf(b A) + bf(c bf(A A)))      P = Q = A   (M x M, symmetric so A A = A At)
-//   BX       X' = bf(bf(a X) + bf(B X))            P = B (M x M), Q = Xt (K x M)
-// BX reads the transposed copy Xt as its second operand and writes both X' and X't, so no
-// operand ever needs a transposing load.  SYRK/SYMPOLY compute only tiles on or above the
-// diagonal and mirror them, which makes the result symmetric bit for bit.
+// The three products of one NS iteration:
+//   SYRK     A  = bf(X Xt)                         P = Q = X   (M x K)           C[i][j] = sum_k P[i][k] Q[j][k]
+//   SYMPOLY  B  = bf(bf(b A) + bf(c bf(A A)))      P = Q = A   (M x M, symmetric so A A = A At)      same
+//   BX       X' = bf(bf(a X) + bf(B X))            P = B (M x M), Q = X (M x K)  C[i][j] = sum_k P[i][k] Q[k][j]
+// SYRK/SYMPOLY contract rows with rows and compute only tiles on or above the diagonal, mirrored in the
+// epilogue, which makes the result symmetric bit for bit.  BX contracts rows of B with columns of X: its Q
+// fragments come out of LDS through the transposing read ds_read_b64_tr_b16, so X is kept in one
+// orientation only.
 //
 // Every bf16 rounding point of the reference's torch expressions
 // (/root/reference/src/lmms_engine/utils/muon_utils.py:149-152) is applied in registers.
 //
-// Operands and results live in the blocked layout of gemm_nt.h (256 x 64 blocks), zero padded
+// Operands and results live in the blocked layout of common.h (256 x 32 blocks), zero padded
 // by the producers to whole tiles, so there is no masking here; the host launcher checks that
 // the shapes it is given are whole tiles before launching.
 #include <type_traits>
@@ -235,6 +235,107 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
     }
 }
 
+// Epilogue of BX.  The accumulators were built with the MFMA operands swapped, so a lane holds 4
+// consecutive columns n of one row m (lane&31 owns row m of its P fragment, registers 4q..4q+3 are columns
+// 8q + 4*(lane>>5) + 0..3 of its Q fragment): 8-byte pieces of rows of X'.  The tile lives in LDS as T[m][n];
+// the a.X term is the same tile of X, loaded into T with coalesced reads, every lane replaces its own pieces
+// by the rounded results in place, and rows of T leave as rows of X' (1 KB contiguous per wave instruction).
+template <int BM, int BN>
+constexpr int epilogue_nn_bytes() { return BM * (BN * 2 + 16); }
+
+template <int BM, int BN, int WGM, int WGN>
+__device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& tc,
+                                            f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], unsigned char* smem) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int S = BN * 2 + 16;           // T row pitch (bytes)
+    constexpr int CPB = BLK_COLS / 8;        // 16-byte chunks per row of a block
+    constexpr int NLE = BM * (BN / 8) / NT;  // 16-byte chunks per thread for a whole tile
+    static_assert((BM * (BN / 8)) % NT == 0 && BN % BLK_COLS == 0, "even split");
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN, hi = lane >> 5;
+    const int m0 = tc.ti * BM, n0 = tc.tj * BN;
+    // chunk c: 16 bytes j of the row piece of row m in column block cbk of the tile; a wave covers 16 rows of
+    // one block = 1 KB contiguous in memory
+    auto tile_chunk = [&](int c, int cb, long& goff, int& loff) {
+        const int j = c % CPB, m = (c / CPB) % BM, cbk = (c / CPB) / BM;
+        goff = panel_offset(m0, cb) + (long)((n0 >> BLK_SHIFT) + cbk) * BLK_ELEMS + m * BLK_COLS + j * 8;
+        loff = m * S + (cbk * CPB + j) * 16;
+    };
+    __syncthreads();  // the operand stages are no longer read
+    const bf16_t* Et = g.Et + tc.bidx * g.strideEt;
+#pragma unroll
+    for (int b = 0; b < NLE; b += 16) {
+        u32x4 ev[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            long goff;
+            int loff;
+            tile_chunk(tid + (b + u) * NT, g.cbEt, goff, loff);
+            if (b + u < NLE) ev[u] = *(const u32x4*)(Et + goff);
+        }
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+            long goff;
+            int loff;
+            tile_chunk(tid + (b + u) * NT, g.cbEt, goff, loff);
+            if (b + u < NLE) *(u32x4*)(smem + loff) = ev[u];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < FM; ++i) {
+        // all LDS reads of a fragment row first (a write in between would serialise them)
+        bf16x4 e[FN][4];
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                e[j][q] = *(const bf16x4*)(smem + (wm * WTM + i * 32 + (lane & 31)) * S +
+                                           (wn * WTN + j * 32 + q * 8 + hi * 4) * 2);
+        bf16x4 o[FN][4];
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    o[j][q][r] = f2bf(rbf(g.s0 * bf2f(e[j][q][r])) + rbf(acc[i][j][q * 4 + r]));
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                *(bf16x4*)(smem + (wm * WTM + i * 32 + (lane & 31)) * S + (wn * WTN + j * 32 + q * 8 + hi * 4) * 2) =
+                    o[j][q];
+    }
+    __syncthreads();
+    bf16_t* C = g.C + tc.bidx * g.strideC;
+#pragma unroll
+    for (int u = 0; u < NLE; ++u) {
+        long goff;
+        int loff;
+        tile_chunk(tid + u * NT, g.cbC, goff, loff);
+        *(u32x4*)(C + goff) = *(const u32x4*)(smem + loff);
+    }
+}
+
+// Transposing LDS read of a Q fragment of BX: the stage holds the k-tile of X as pieces of 32 columns,
+// [piece][k][32 columns] with 64-byte rows.  In a group of 16 lanes, lane j = 4r+s addresses row k+r, columns
+// 4s..4s+3 of the group's 16 columns and lane i = 4s+e receives rows k..k+3 of column 4s+e; the second read takes
+// rows k+4..k+7.  Lanes 16..31 take the upper 16 columns and lanes 32..63 rows k+8.., which is the MFMA operand
+// layout (lane l: row l%32 of the fragment, eight consecutive k from 8*(l/32)).  q points at row k of the piece
+// plus qt_lane_offset(lane).
+__device__ __forceinline__ int qt_lane_offset(int lane) {
+    const int grp = lane >> 4, i16 = lane & 15;
+    return ((grp >> 1) * 8 + (i16 >> 2)) * 64 + (grp & 1) * 32 + (i16 & 3) * 8;
+}
+__device__ __forceinline__ bf16x8 lds_read_qt(const unsigned char* q) {
+    const s16x4 lo = lds_read_tr16(q), hi4 = lds_read_tr16(q + 4 * 64);
+    const s16x8 t = {lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+    return *(const bf16x8*)&t;
+}
+
 // ---- kernel 1: 64-column k-tiles in two LDS stages, one barrier per k-tile -------------------
 // Operand panels go from global memory straight into LDS (global_load_lds_dwordx4): one wave
 // instruction fills 1 KB of LDS in lane order, i.e. 8 rows of 128 bytes, so the XOR swizzle
@@ -270,13 +371,17 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const TileCoord tc = decode_tile<EPI>(g);
+    constexpr bool QT = EPI == EPI_BX;  // Q is X itself, rows = reduction index
     const int kb = g.kdim / BLK_COLS;
     const bf16_t* Pb = g.P + tc.bidx * g.strideP + panel_offset(tc.ti * BM, kb);
-    const bf16_t* Qb = g.Q + tc.bidx * g.strideQ + panel_offset(tc.tj * BN, kb);
+    const bf16_t* Qb = g.Q + tc.bidx * g.strideQ +
+                       (QT ? (long)(tc.tj * BN >> BLK_SHIFT) * BLK_ELEMS : panel_offset(tc.tj * BN, kb));
 
     const int drow = lane >> 3;
     const bf16_t* pa = Pb + (wave * 8 * LA + drow) * BLK_COLS;
-    const bf16_t* pb = Qb + (wave * 8 * LB + drow) * BLK_COLS;
+    // BX: a k-tile of Q is BN/32 pieces of 64 rows x 32 columns, each a contiguous 4 KB run of one block;
+    // load instruction t of the tile (1 KB) is the quarter t%4 of piece t/4, in lane order
+    const bf16_t* pb = QT ? Qb + (lane >> 2) * BLK_COLS + (lane & 3) * 8 : Qb + (wave * 8 * LB + drow) * BLK_COLS;
     const int lds_a = wave * 8 * LA * ROW_BYTES;
     const int lds_b = A_BYTES + wave * 8 * LB * ROW_BYTES;
     // element offset of the 16-byte chunk this lane fetches inside a row of the 64-column k-tile, as an offset
@@ -292,6 +397,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
             const long ch = ((wave * LA + n) & 1) ? ch_odd : ch_even;
             __builtin_amdgcn_global_load_lds((glb_void_ptr)(pa + (long)kt * KT_BLOCKS * BLK_ELEMS + n * 8 * BLK_COLS + ch),
                                              (lds_void_ptr)(s + lds_a + n * 8 * ROW_BYTES), 16, 0, 0);
+        } else if (QT) {
+            const int i = n - LA, t = wave * LB + i, k0 = kt * 64;
+            const long off = ((long)(k0 >> 8) * g.cbQ + (t >> 2)) * BLK_ELEMS + ((k0 & 255) + (t & 3) * 16) * BLK_COLS;
+            __builtin_amdgcn_global_load_lds((glb_void_ptr)(pb + off), (lds_void_ptr)(s + lds_b + i * 8 * ROW_BYTES), 16, 0, 0);
         } else {
             const int i = n - LA;
             const long ch = ((wave * LB + i) & 1) ? ch_odd : ch_even;
@@ -310,17 +419,22 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
 
     const int sw = (lane >> 1) & 7, hi = lane >> 5;
     const int a_off = (wm * WTM + (lane & 31)) * ROW_BYTES;
-    const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROW_BYTES;
+    const int b_off = QT ? A_BYTES + (wn * WTN / 32) * 4096 + qt_lane_offset(lane)
+                         : A_BYTES + (wn * WTN + (lane & 31)) * ROW_BYTES;
 
-    bf16x8 fr[2][NRD];  // fragment double buffer: [0..FM) rows of P, [FM..NRD) rows of Q
+    bf16x8 fr[2][NRD];  // fragment double buffer: [0..FM) rows of P, [FM..NRD) rows (BX: columns) of Q
     auto read_one = [&](int buf, int n, const unsigned char* st, int ks) {
         const int co = (((ks << 1) | hi) ^ sw) << 4;
         if (n < FM) fr[buf][n] = *(const bf16x8*)(st + a_off + n * 32 * ROW_BYTES + co);
+        else if (QT) fr[buf][n] = lds_read_qt(st + b_off + (n - FM) * 4096 + ks * 16 * 64);
         else fr[buf][n] = *(const bf16x8*)(st + b_off + (n - FM) * 32 * ROW_BYTES + co);
     };
     auto mfma_one = [&](int buf, int idx) {
         const int i = idx / FN, j = idx % FN;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[buf][i], fr[buf][FM + j], acc[i][j], 0, 0, 0);
+        if (QT)  // operands swapped: a lane then holds 4 consecutive columns of one row of the tile
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[buf][FM + j], fr[buf][i], acc[i][j], 0, 0, 0);
+        else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[buf][i], fr[buf][FM + j], acc[i][j], 0, 0, 0);
     };
 
     const int nk = g.kdim / 64;
@@ -376,156 +490,11 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
         }
     }
     WAIT_VM(0);  // the dummy loads of the last two tails must not land in the epilogue's tile
-    epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN>(g, tc, acc, smem);
+    else epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 }
 
-// ---- kernel 2: 32-column k-tiles in four LDS stages -------------------------------------------
-// The L1 -> LDS path moves 64 B/clk per CU, so feeding a 256x256 tile keeps it busy half of
-// the time; when the loads of a k-tile are issued in one burst (kernel 1) every wave of the CU
-// queues on the one address path and its MFMAs starve behind the blocked load.  Four stages of
-// 32 columns leave a stage free for a whole k-tile, so the loads are spread evenly.  Timeline of
-// wave w for k-tile t (stage t&3, two k-steps):
-//   phase A: MFMAs of k-step 0 | fragment reads of k-step 1 | B-half loads of k-tile t+3
-//   wait own reads; wait own loads of k-tile t+1; barrier   (stage t&3 is now free)
-//   phase B: MFMAs of k-step 1 | fragment reads of k-tile t+1 step 0 | A-half loads of k-tile t+4
-// LDS rows are 64 B (4 chunks); chunk c of row r sits at position c ^ ((r>>2)&3).  K-tile t is
-// columns 32t.. of the panel.
-template <int BM, int BN, int WGM, int WGN, int EPI>
-__global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe4_kernel(const GemmArgs g) {
-    constexpr int NW = WGM * WGN;
-    constexpr int BK4 = 32, ROWB = 64;
-    constexpr int WTM = BM / WGM, WTN = BN / WGN;
-    constexpr int FM = WTM / 32, FN = WTN / 32;
-    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
-    constexpr int LA = BM / 16 / NW, LB = BN / 16 / NW;  // 1 KB loads (16 rows) per wave per k-tile
-    constexpr int NMF = FM * FN, NRD = FM + FN;
-    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "dma split");
-    // Slot plan of one phase (NMF MFMAs, NRD fragment reads, L loads): the loads sit behind every
-    // (NMF/L)-th MFMA so that the waves of the CU, which run in lockstep, hand the one L1
-    // address path a few loads per NMF/L MFMAs instead of all of them back to back; the reads fill
-    // the other slots from the front.
-    constexpr int LSP_A = NMF / LB > 0 ? NMF / LB : 1, LSP_B = NMF / LA > 0 ? NMF / LA : 1;
-    constexpr int RPS_A = (NRD + (NMF - NMF / LSP_A) - 1) / (NMF - NMF / LSP_A > 0 ? NMF - NMF / LSP_A : 1);
-    constexpr int RPS_B = (NRD + (NMF - NMF / LSP_B) - 1) / (NMF - NMF / LSP_B > 0 ? NMF - NMF / LSP_B : 1);
-    static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
-
-    extern __shared__ __align__(16) unsigned char smem[];
-
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / WGN, wn = wave % WGN;
-    const TileCoord tc = decode_tile<EPI>(g);
-    const int kb = g.kdim / BLK_COLS;
-    const bf16_t* Pb = g.P + tc.bidx * g.strideP + panel_offset(tc.ti * BM, kb);
-    const bf16_t* Qb = g.Q + tc.bidx * g.strideQ + panel_offset(tc.tj * BN, kb);
-
-    // lane L of a load lands on row L>>2, position L&3 and so fetches chunk (L&3)^((L>>4)&3)
-    const int drow = lane >> 2;
-    const int dch = ((lane & 3) ^ ((lane >> 4) & 3)) * 8;
-    const bf16_t* pa = Pb + (wave * 16 * LA + drow) * BLK_COLS + dch;
-    const bf16_t* pb = Qb + (wave * 16 * LB + drow) * BLK_COLS + dch;
-    const int lds_a = wave * 16 * LA * ROWB;
-    const int lds_b = A_BYTES + wave * 16 * LB * ROWB;
-    const int nk = g.kdim / BK4;
-
-    auto ktile_offset = [&](int kt) {  // kt may run past the end: re-load the last k-tile
-        const int k0 = (kt < nk ? kt : nk - 1) * BK4;
-        return (long)(k0 >> BLK_SHIFT) * BLK_ELEMS + (k0 & (BLK_COLS - 1));
-    };
-    auto issue_a = [&](int n, int kt) {
-        __builtin_amdgcn_global_load_lds((glb_void_ptr)(pa + ktile_offset(kt) + n * 16 * BLK_COLS),
-                                         (lds_void_ptr)(smem + (kt & 3) * STAGE + lds_a + n * 16 * ROWB), 16, 0, 0);
-    };
-    auto issue_b = [&](int n, int kt) {
-        __builtin_amdgcn_global_load_lds((glb_void_ptr)(pb + ktile_offset(kt) + n * 16 * BLK_COLS),
-                                         (lds_void_ptr)(smem + (kt & 3) * STAGE + lds_b + n * 16 * ROWB), 16, 0, 0);
-    };
-
-    f32x16 acc[FM][FN];
-#pragma unroll
-    for (int i = 0; i < FM; ++i)
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-
-    const int sw = (lane >> 2) & 3, hi = lane >> 5;
-    const int a_off = (wm * WTM + (lane & 31)) * ROWB;
-    const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROWB;
-
-    bf16x8 fr[2][NRD];
-    auto read_one = [&](int buf, int n, const unsigned char* st, int ks) {
-        const int co = (((ks << 1) | hi) ^ sw) << 4;
-        if (n < FM) fr[buf][n] = *(const bf16x8*)(st + a_off + n * 32 * ROWB + co);
-        else fr[buf][n] = *(const bf16x8*)(st + b_off + (n - FM) * 32 * ROWB + co);
-    };
-    auto mfma_one = [&](int buf, int idx) {
-        const int i = idx / FN, j = idx % FN;
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[buf][i], fr[buf][FM + j], acc[i][j], 0, 0, 0);
-    };
-
-    // prologue: k-tiles 0..2 and the A half of k-tile 3
-#pragma unroll
-    for (int t = 0; t < 3; ++t) {
-#pragma unroll
-        for (int n = 0; n < LA; ++n) issue_a(n, t);
-#pragma unroll
-        for (int n = 0; n < LB; ++n) issue_b(n, t);
-    }
-#pragma unroll
-    for (int n = 0; n < LA; ++n) issue_a(n, 3);
-    WAIT_VM(2 * (LA + LB) + LA);
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-#pragma unroll
-    for (int n = 0; n < NRD; ++n) read_one(0, n, smem, 0);
-
-    for (int kt = 0; kt < nk; ++kt) {
-        const unsigned char* st = smem + (kt & 3) * STAGE;
-        const unsigned char* stn = smem + ((kt + 1) & 3) * STAGE;
-        // phase A
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int idx = 0; idx < NMF; ++idx) {
-            mfma_one(0, idx);
-            __builtin_amdgcn_sched_barrier(0);
-            if ((idx + 1) % LSP_A == 0) {
-                if (idx / LSP_A < LB) issue_b(idx / LSP_A, kt + 3);
-            } else {
-                const int r0 = (idx - idx / LSP_A) * RPS_A;
-#pragma unroll
-                for (int u = 0; u < RPS_A; ++u)
-                    if (r0 + u < NRD) read_one(1, r0 + u, st, 1);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        // own reads of this stage are complete, own loads of k-tile kt+1 have landed
-        WAIT_LGKM0();
-        WAIT_VM(2 * (LA + LB));
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
-        // phase B
-#pragma unroll
-        for (int idx = 0; idx < NMF; ++idx) {
-            mfma_one(1, idx);
-            __builtin_amdgcn_sched_barrier(0);
-            if ((idx + 1) % LSP_B == 0) {
-                if (idx / LSP_B < LA) issue_a(idx / LSP_B, kt + 4);
-            } else {
-                const int r0 = (idx - idx / LSP_B) * RPS_B;
-#pragma unroll
-                for (int u = 0; u < RPS_B; ++u)
-                    if (r0 + u < NRD) read_one(0, r0 + u, stn, 0);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
-    epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
-}
-
-// ---- kernel 3: eight waves in two groups that alternate between memory and MFMA phases --------
+// ---- kernel 2: eight waves in two groups that alternate between memory and MFMA phases --------
 // Every wave runs the same loop  { M(t): read its fragments of k-tile t from LDS, issue its
 // share of the loads of k-tile t+3, wait;  barrier;  C(t): FM*FN*2 MFMAs;  barrier }  over
 // 32-column k-tiles in four LDS stages, but waves 4..7 enter it one barrier later than waves
@@ -553,9 +522,11 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2;
     const int wm = wave / WGN, wn = wave % WGN;
+    constexpr bool QT = EPI == EPI_BX;  // Q is X itself, rows = reduction index
     const int kb = g.kdim / BLK_COLS;
     const bf16_t* Pb = uniform_ptr(g.P + tc.bidx * g.strideP + panel_offset(tc.ti * BM, kb));
-    const bf16_t* Qb = uniform_ptr(g.Q + tc.bidx * g.strideQ + panel_offset(tc.tj * BN, kb));
+    const bf16_t* Qb = uniform_ptr(g.Q + tc.bidx * g.strideQ +
+                                   (QT ? (long)(tc.tj * BN >> BLK_SHIFT) * BLK_ELEMS : panel_offset(tc.tj * BN, kb)));
 
     // Loads: a wave-uniform base pointer (advanced along k with scalar adds) plus a 32-bit byte
     // offset per lane, so that no vector ALU instruction is needed per load: in the memory phase
@@ -565,8 +536,14 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     unsigned offa[LA], offb[LB];
 #pragma unroll
     for (int n = 0; n < LA; ++n) offa[n] = (unsigned)(((wave * 16 * LA + n * 16 + drow) * BLK_COLS + dch) * 2);
+    // BX: a k-tile of Q is BN/32 pieces of 32 rows x 32 columns, each a contiguous 2 KB run of one block; load
+    // instruction t of the tile (1 KB) is the half t%2 of piece t/2, in lane order
 #pragma unroll
-    for (int n = 0; n < LB; ++n) offb[n] = (unsigned)(((wave * 16 * LB + n * 16 + drow) * BLK_COLS + dch) * 2);
+    for (int n = 0; n < LB; ++n) {
+        const int t = wave * LB + n;
+        offb[n] = QT ? (unsigned)(((t >> 1) * BLK_ELEMS + ((t & 1) * 16 + drow) * BLK_COLS + (lane & 3) * 8) * 2)
+                     : (unsigned)(((wave * 16 * LB + n * 16 + drow) * BLK_COLS + dch) * 2);
+    }
     const int lds_a = wave * 16 * LA * ROWB;
     const int lds_b = A_BYTES + wave * 16 * LB * ROWB;
     const int nk = g.kdim / BK4;
@@ -584,7 +561,7 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
         const int k0 = (kt < nk ? kt : nk - 1) * BK4;
         const long koff = (long)(k0 >> BLK_SHIFT) * BLK_ELEMS + (k0 & (BLK_COLS - 1));
         const char* ba = (const char*)(Pb + koff);
-        const char* bb = (const char*)(Qb + koff);
+        const char* bb = (const char*)(Qb + (QT ? (long)(k0 >> 8) * g.cbQ * BLK_ELEMS + (k0 & 255) * BLK_COLS : koff));
         const unsigned st = lds_base + (kt & 3) * STAGE;
 #pragma unroll
         for (int n = 0; n < LA; ++n) dma(ba, offa[n], st + lds_a + n * 16 * ROWB);
@@ -623,7 +600,8 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             ra[ks][half] = smem + half * 2 * STAGE + a_off + co;
-            rb[ks][half] = smem + half * 2 * STAGE + b_off + co;
+            rb[ks][half] = QT ? smem + half * 2 * STAGE + A_BYTES + (wn * WTN / 32) * 2048 + ks * 16 * 64 + qt_lane_offset(lane)
+                              : smem + half * 2 * STAGE + b_off + co;
         }
     }
     auto body = [&](int kt, auto stage_c) {
@@ -636,8 +614,10 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
             for (int i = 0; i < FM; ++i)
                 fa[ks][i] = *(const bf16x8*)(ra[ks][SIDX >> 1] + (SIDX & 1) * STAGE + i * 32 * ROWB);
 #pragma unroll
-            for (int j = 0; j < FN; ++j)
-                fb[ks][j] = *(const bf16x8*)(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 32 * ROWB);
+            for (int j = 0; j < FN; ++j) {
+                if (QT) fb[ks][j] = lds_read_qt(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 2048);
+                else fb[ks][j] = *(const bf16x8*)(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 32 * ROWB);
+            }
         }
         issue_tile(kt + 3);
         WAIT_LGKM0();
@@ -653,8 +633,12 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
 #pragma unroll
             for (int i = 0; i < FM; ++i)
 #pragma unroll
-                for (int j = 0; j < FN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < FN; ++j) {
+                    if (QT)  // operands swapped: a lane then holds 4 consecutive columns of one row of the tile
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+                    else
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
+                }
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
@@ -670,7 +654,8 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     }
     if (!grp) __builtin_amdgcn_s_barrier();
     WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
-    epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN>(g, tc, acc, smem);
+    else epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
 }
 
 template <int BM, int BN, int WGM, int WGN, int EPI>
@@ -701,12 +686,12 @@ __global__ void __launch_bounds__(512) gemm_nt_pp_tail_kernel(const GemmArgs g) 
 
 template <int BM, int BN, int WGM, int WGN, int EPI, int FEED>
 hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
-    constexpr int stages = 2 * (BM + BN) * ROW_BYTES, epi = epilogue_bytes<BM, BN>();
+    constexpr int stages = 2 * (BM + BN) * ROW_BYTES;
+    constexpr int epi = EPI == EPI_BX ? epilogue_nn_bytes<BM, BN>() : epilogue_bytes<BM, BN>();
     constexpr int smem = stages > epi ? stages : epi;
     static bool configured = false;  // per instantiation; the attribute is idempotent
     void (*kern)(const GemmArgs);
-    if constexpr (FEED == 2) kern = gemm_nt_pp_kernel<BM, BN, WGM, WGN, EPI>;
-    else if constexpr (FEED == 1) kern = gemm_nt_pipe4_kernel<BM, BN, WGM, WGN, EPI>;
+    if constexpr (FEED == 1) kern = gemm_nt_pp_kernel<BM, BN, WGM, WGN, EPI>;
     else kern = gemm_nt_pipe_kernel<BM, BN, WGM, WGN, EPI>;
     if (!configured) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -722,9 +707,7 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
     switch (cfg) {
         case GEMM_CFG_128_PIPE: return launch_one<128, 128, 2, 2, EPI, 0>(g, nblocks, stream);
         case GEMM_CFG_256_PIPE: return launch_one<256, 256, 2, 4, EPI, 0>(g, nblocks, stream);
-        case GEMM_CFG_128_PIPE4: return launch_one<128, 128, 2, 2, EPI, 1>(g, nblocks, stream);
-        case GEMM_CFG_256_W4_PIPE4: return launch_one<256, 256, 2, 2, EPI, 1>(g, nblocks, stream);
-        case GEMM_CFG_256_PINGPONG: return launch_one<256, 256, 2, 4, EPI, 2>(g, nblocks, stream);
+        case GEMM_CFG_256_PINGPONG: return launch_one<256, 256, 2, 4, EPI, 1>(g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -733,10 +716,8 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
 
 int gemm_cfg_tile(int cfg) {
     switch (cfg) {
-        case GEMM_CFG_128_PIPE:
-        case GEMM_CFG_128_PIPE4: return 128;
+        case GEMM_CFG_128_PIPE: return 128;
         case GEMM_CFG_256_PIPE:
-        case GEMM_CFG_256_W4_PIPE4:
         case GEMM_CFG_256_PINGPONG: return 256;
         default: return 0;
     }
@@ -744,7 +725,8 @@ int gemm_cfg_tile(int cfg) {
 
 template <int EPI>
 hipError_t launch_pp_tail(GemmArgs g, int nblocks, int rest, hipStream_t stream) {
-    constexpr int stages = 2 * (256 + 256) * ROW_BYTES, epi = epilogue_bytes<256, 256>();
+    constexpr int stages = 2 * (256 + 256) * ROW_BYTES;
+    constexpr int epi = EPI == EPI_BX ? epilogue_nn_bytes<256, 256>() : epilogue_bytes<256, 256>();
     constexpr int smem = stages > epi ? stages : epi;  // the 128-tiles need less of both
     static bool configured = false;
     auto kern = gemm_nt_pp_tail_kernel<EPI>;

@@ -82,7 +82,7 @@ def matmul_transpose_assign(d_in: Tensor, d_out: Tensor) -> None:
         raise TypeError(f"the MI355X kernel multiplies bfloat16 operands, got {d_in.dtype}")
     M, K = d_in.shape
     tile = 256 if (M % 256 == 0 and M >= 512) else 128
-    cfg = _abi.CFG_AUTO if tile == 256 else _abi.CFG_128_PIPE4
+    cfg = _abi.CFG_AUTO if tile == 256 else _abi.CFG_128_PIPE
     Mp, Kp = -(-M // tile) * tile, -(-K // tile) * tile
     lib = _abi.lib()
     with torch.cuda.device(d_in.device):

@@ -47,7 +47,7 @@ def _assert_product_close(got, ref64, absprod):
     assert not bad.any(), f"{int(bad.sum())} elements outside one bf16 ulp"
 
 
-CFGS = list(range(5))
+CFGS = list(range(3))
 
 
 def _pack(env, t):
@@ -141,40 +141,24 @@ def test_sympoly_rounding_points(env, cfg):
 
 
 @pytest.mark.parametrize("cfg", CFGS)
-@pytest.mark.parametrize("outputs", ["both", "x", "xt"])
-def test_bx_axpy_rounding_points(env, cfg, outputs):
-    print(f"bx cfg={cfg} outputs={outputs}", flush=True)
+@pytest.mark.parametrize("M,K", [(256, 768), (512, 256)])
+def test_bx_axpy_rounding_points(env, cfg, M, K):
+    print(f"bx cfg={cfg} M={M} K={K}", flush=True)
     O = env["O"]
     g = torch.Generator().manual_seed(30 + cfg)
-    M, K, batch = 256, 768, 2
+    batch = 2
     X = (torch.randn(batch, M, K, generator=g) / 16).bfloat16()
     Bm = (torch.randn(batch, M, M, generator=g) / 16).bfloat16()
     Bm = torch.triu(Bm) + torch.triu(Bm, 1).mT  # the kernel is specified for symmetric B
     dev = env["dev"]
-    Xo, XTo = _blocked_nan(env, batch, M, K), _blocked_nan(env, batch, K, M)
-    XT = _pack(env, X.mT.contiguous().to(dev))
-    Bb = _pack(env, Bm.to(dev))
+    Xb, Bb, Xo = _pack(env, X.to(dev)), _pack(env, Bm.to(dev)), _blocked_nan(env, batch, M, K)
     a = O.NS_COEFFS[0]
-    env["abi"].check(env["lib"].muon_hip_bx_axpy_bf16(
-        Bb.data_ptr(), XT.data_ptr(), Xo.data_ptr() if outputs != "xt" else None,
-        XTo.data_ptr() if outputs != "x" else None, M, K, batch, a, cfg, 0))
-    Xo, XTo = _unpack(env, Xo, batch, M, K), _unpack(env, XTo, batch, K, M)
+    env["abi"].check(env["lib"].muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, a, cfg, 0))
+    Xo = _unpack(env, Xo, batch, M, K)
     for i in range(batch):
         ref = (O.bf(X[i].float() * O._f32(a)) + O.bf(Bm[i].float() @ X[i].float())).bfloat16()
-        if outputs != "xt":
-            got = Xo[i]
-            assert (got != ref).float().mean().item() < 2e-2
-            assert rel_fro(got, ref) < 4e-3
-        else:
-            assert torch.isnan(Xo).all()
-        if outputs != "x":
-            got = XTo[i].mT
-            assert (got != ref).float().mean().item() < 2e-2
-            assert rel_fro(got, ref) < 4e-3
-        else:
-            assert torch.isnan(XTo).all()
-    if outputs == "both":
-        assert torch.equal(Xo, XTo.mT)
+        assert (Xo[i] != ref).float().mean().item() < 2e-2
+        assert rel_fro(Xo[i], ref) < 4e-3
 
 
 def test_split_tail_is_bitwise_the_plain_kernel(env):
@@ -195,17 +179,15 @@ def test_split_tail_is_bitwise_the_plain_kernel(env):
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
     assert torch.equal(outs[0][0], outs[0][0].mT) and not torch.isnan(outs[0][1]).any()
     M, K, batch = 1024, 512, 33
-    XT = _pack(env, (torch.randn(batch, K, M, generator=g) / 16).bfloat16().to(dev))
+    Xb = _pack(env, (torch.randn(batch, M, K, generator=g) / 16).bfloat16().to(dev))
     Bm = (torch.randn(batch, M, M, generator=g) / 16).bfloat16()
     Bb = _pack(env, (torch.triu(Bm) + torch.triu(Bm, 1).mT).to(dev))
     outs = []
     for cfg in (abi.CFG_256_PINGPONG, abi.CFG_256_PIPE):
-        Xo, XTo = _blocked_nan(env, batch, M, K), _blocked_nan(env, batch, K, M)
-        abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), XT.data_ptr(), Xo.data_ptr(), XTo.data_ptr(), M, K, batch,
-                                            O.NS_COEFFS[0], cfg, 0))
-        outs.append((_unpack(env, Xo, batch, M, K), _unpack(env, XTo, batch, K, M)))
-    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
-    assert torch.equal(outs[0][0], outs[0][1].mT) and not torch.isnan(outs[0][0]).any()
+        Xo = _blocked_nan(env, batch, M, K)
+        abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, O.NS_COEFFS[0], cfg, 0))
+        outs.append(_unpack(env, Xo, batch, M, K))
+    assert torch.equal(outs[0], outs[1]) and not torch.isnan(outs[0]).any()
 
 
 def test_gemm_entry_points_reject_bad_shapes(env):
@@ -217,7 +199,8 @@ def test_gemm_entry_points_reject_bad_shapes(env):
     assert lib.muon_hip_syrk_bf16(None, x.data_ptr(), 256, 256, 1, 0, 0) == -1
     assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 256, 256, 1, 99, 0) == -1
     with pytest.raises(abi.MuonHipError):
-        abi.check(lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), None, None, 256, 256, 1, 1.0, 0, 0))
+        abi.check(lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), None, 256, 256, 1, 1.0, 0, 0))
+    assert lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), x.data_ptr(), 256, 256, 1, 1.0, 0, 0) == -1  # in place
 
 
 NS_SHAPES = [(64, 160), (160, 64), (33, 47), (100, 300), (300, 100), (128, 896), (896, 128), (256, 256), (512, 1024)]
