@@ -366,6 +366,26 @@ def test_full_step_bf16_params(env, momentum_dtype):
         assert wp <= 4e-3  # a few bf16 roundings of p differ where the update differs
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_full_step_ragged_and_tall_shapes(env, dtype):
+    """Shapes that are not whole tiles, not multiples of 8 and taller than wide (the update is then the transpose
+    of the Newton-Schulz operand and goes through the transposing kernels), two steps each."""
+    names = ["tall_odd", "wide_odd", "tall", "tall_vec", "square_odd", "thin"]
+    shapes = [(53, 37), (37, 53), (300, 100), (640, 256), (129, 129), (1000, 8)]
+    gen = torch.Generator().manual_seed(17)
+    weights = [(n, 0.02 * torch.randn(*s, generator=gen)) for n, s in zip(names, shapes)]
+    opt, orc, gp, cp = _build_opts(env, weights, MUON_HP, dtype, momentum_dtype=torch.float32 if dtype == torch.bfloat16 else None)
+    for step in range(2):
+        grads = [1e-3 * torch.randn(*s, generator=gen) for s in shapes]
+        wu, wm, wp = _check_step(opt, orc, gp, cp, grads, dtype, None)
+        print(f"ragged {dtype} step {step}: update {wu:.3e} momentum {wm:.3e} param {wp:.3e}", flush=True)
+        assert wm <= MOM_TOL
+        if dtype == torch.float32:
+            assert wu <= NS_TOL and wp <= 2e-3  # params move by lr*update; 2e-2 of that relative to ||p||
+        else:
+            assert wp <= 4e-3
+
+
 def test_grouped_equals_per_matrix_bitwise(env):
     mu = env["mu"]
     weights, grads = make_param_set(dict(QWEN25_05B, q=(256, 256), o=(256, 256), k=(128, 256), v=(128, 256),
