@@ -105,12 +105,13 @@ __device__ __forceinline__ long panel_offset(int row0, int cb) {
 // ---- epilogue ------------------------------------------------------------------------------
 // One LDS copy of the tile, both output orientations written as 16-byte vectors.  The tile
 // lives in LDS as Tt[n][m] (n = local column, m = local row of the accumulator tile), the
-// orientation of Ct and of the elementwise source Et: Et is loaded into it with coalesced reads,
-// every lane replaces its own 8-byte pieces (4 consecutive m of one n, exactly what an
-// accumulator lane holds: lane&31 owns column n, registers 4q..4q+3 are rows 8q + 4*(lane>>5) +
-// 0..3) by the rounded results, and after one barrier rows of Tt leave as rows of Ct, while
-// rows of C are gathered with ds_read_b64_tr_b16: in a group of 16 lanes, lane i receives
-// element i%4 of the 8-byte pieces addressed by lanes i/4, 4+i/4, 8+i/4, 12+i/4.
+// orientation of Ct and of the elementwise source Et.  Every lane writes its rounded accumulators
+// as 8-byte pieces (4 consecutive m of one n, exactly what an accumulator lane holds: lane&31 owns
+// column n, registers 4q..4q+3 are rows 8q + 4*(lane>>5) + 0..3); after one barrier rows of Tt
+// leave as rows of Ct (SYMPOLY adds the b.A term there, from pieces of Et that each thread loaded
+// into registers before the accumulators were written, and puts the sums back), while rows of C
+// are gathered with ds_read_b64_tr_b16: in a group of 16 lanes, lane i receives element i%4 of the
+// 8-byte pieces addressed by lanes i/4, 4+i/4, 8+i/4, 12+i/4.
 // Diagonal tiles of the symmetric kernels write the full tile once: acc(i,j) and acc(j,i) are
 // sums of the same exact products in the same order.
 template <int BM, int BN>
@@ -144,73 +145,54 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
         goff = panel_offset(n0, cb) + (long)((m0 >> BLK_SHIFT) + cbk) * BLK_ELEMS + n * BLK_COLS + j * 8;
         loff = n * S + (cbk * CPB + j) * 16;
     };
-    __syncthreads();  // the operand stages are no longer read
-    if (EPI != EPI_SYRK) {
+    // SYMPOLY: this thread's 16-byte pieces of the b.A term, in the layout of the Ct pass, go to registers
+    // first, so that the loads are in flight while the accumulators are rounded into LDS
+    bf16x8 ev[EPI == EPI_SYMPOLY ? NLE : 1];
+    if (EPI == EPI_SYMPOLY) {
         const bf16_t* Et = g.Et + tc.bidx * g.strideEt;
 #pragma unroll
-        for (int b = 0; b < NLE; b += 16) {
-            u32x4 ev[16];
-#pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                long goff;
-                int loff;
-                tile_chunk(tid + (b + u) * NT, g.cbEt, goff, loff);
-                if (b + u < NLE) ev[u] = *(const u32x4*)(Et + goff);
-            }
-#pragma unroll
-            for (int u = 0; u < 16; ++u) {
-                long goff;
-                int loff;
-                tile_chunk(tid + (b + u) * NT, g.cbEt, goff, loff);
-                if (b + u < NLE) *(u32x4*)(smem + loff) = ev[u];
-            }
+        for (int u = 0; u < NLE; ++u) {
+            long goff;
+            int loff;
+            tile_chunk(tid + u * NT, g.cbEt, goff, loff);
+            ev[u] = *(const bf16x8*)(Et + goff);
         }
-        __syncthreads();
     }
+    __syncthreads();  // the operand stages are no longer read
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        // all LDS reads of a fragment row first: in one loop the compiler must assume that each
-        // write may alias the next read and the chain becomes one LDS latency per item
-        bf16x4 e[FN][4];
-        if (EPI != EPI_SYRK) {
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    e[j][q] = *(const bf16x4*)(smem + (wn * WTN + j * 32 + (lane & 31)) * S +
-                                               (wm * WTM + i * 32 + q * 8 + hi * 4) * 2);
-        }
-        bf16x4 o[FN][4];
-#pragma unroll
-        for (int j = 0; j < FN; ++j) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float v = rbf(acc[i][j][q * 4 + r]);
-                    if (EPI == EPI_SYMPOLY) v = rbf(rbf(g.s0 * bf2f(e[j][q][r])) + rbf(g.s1 * v));
-                    if (EPI == EPI_BX) v = rbf(rbf(g.s0 * bf2f(e[j][q][r])) + v);
-                    o[j][q][r] = f2bf(v);
-                }
-            }
-        }
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-                *(bf16x4*)(smem + (wn * WTN + j * 32 + (lane & 31)) * S + (wm * WTM + i * 32 + q * 8 + hi * 4) * 2) =
-                    o[j][q];
-    }
+            for (int q = 0; q < 4; ++q) {
+                bf16x4 o;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    float v = rbf(acc[i][j][q * 4 + r]);
+                    if (EPI == EPI_SYMPOLY) v = g.s1 * v;
+                    o[r] = f2bf(v);
+                }
+                *(bf16x4*)(smem + (wn * WTN + j * 32 + (lane & 31)) * S + (wm * WTM + i * 32 + q * 8 + hi * 4) * 2) = o;
+            }
     __syncthreads();
-    if (g.Ct) {
+    {
+        // rows of Tt leave as rows of Ct; SYMPOLY adds the rounded b.A term here and, when the tile itself is
+        // gathered from LDS afterwards, puts the finished pieces back
         bf16_t* Ct = g.Ct + tc.bidx * g.strideCt;
 #pragma unroll
         for (int u = 0; u < NLE; ++u) {
             long goff;
             int loff;
             tile_chunk(tid + u * NT, g.cbCt, goff, loff);
-            *(u32x4*)(Ct + goff) = *(const u32x4*)(smem + loff);
+            bf16x8 t = *(const bf16x8*)(smem + loff);
+            if (EPI == EPI_SYMPOLY) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) t[k] = f2bf(rbf(g.s0 * bf2f(ev[u][k])) + bf2f(t[k]));
+                if (!diag) *(bf16x8*)(smem + loff) = t;
+            }
+            if (g.Ct) *(bf16x8*)(Ct + goff) = t;
         }
+        if (EPI == EPI_SYMPOLY && !diag) __syncthreads();
     }
     if (g.C && !diag) {
         // lane j = 4r+s of a group addresses row n + 8s + r (then + 4), pieces m = 4c..4c+3: lane i = 4s+e
@@ -237,9 +219,11 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
 
 // Epilogue of BX.  The accumulators were built with the MFMA operands swapped, so a lane holds 4
 // consecutive columns n of one row m (lane&31 owns row m of its P fragment, registers 4q..4q+3 are columns
-// 8q + 4*(lane>>5) + 0..3 of its Q fragment): 8-byte pieces of rows of X'.  The tile lives in LDS as T[m][n];
-// the a.X term is the same tile of X, loaded into T with coalesced reads, every lane replaces its own pieces
-// by the rounded results in place, and rows of T leave as rows of X' (1 KB contiguous per wave instruction).
+// 8q + 4*(lane>>5) + 0..3 of its Q fragment): 8-byte pieces of rows of X'.  Every thread first issues the
+// loads of its share of the a.X tile (16-byte pieces of rows, the layout of the output pass) into registers,
+// then the rounded accumulators go to LDS as T[m][n] while those loads are in flight; after one barrier each
+// thread reads its pieces of T, adds the rounded a.X term and stores rows of X' (1 KB contiguous per wave
+// instruction).
 template <int BM, int BN>
 constexpr int epilogue_nn_bytes() { return BM * (BN * 2 + 16); }
 
@@ -263,52 +247,27 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
         goff = panel_offset(m0, cb) + (long)((n0 >> BLK_SHIFT) + cbk) * BLK_ELEMS + m * BLK_COLS + j * 8;
         loff = m * S + (cbk * CPB + j) * 16;
     };
-    __syncthreads();  // the operand stages are no longer read
     const bf16_t* Et = g.Et + tc.bidx * g.strideEt;
+    bf16x8 ev[NLE];
 #pragma unroll
-    for (int b = 0; b < NLE; b += 16) {
-        u32x4 ev[16];
-#pragma unroll
-        for (int u = 0; u < 16; ++u) {
-            long goff;
-            int loff;
-            tile_chunk(tid + (b + u) * NT, g.cbEt, goff, loff);
-            if (b + u < NLE) ev[u] = *(const u32x4*)(Et + goff);
-        }
-#pragma unroll
-        for (int u = 0; u < 16; ++u) {
-            long goff;
-            int loff;
-            tile_chunk(tid + (b + u) * NT, g.cbEt, goff, loff);
-            if (b + u < NLE) *(u32x4*)(smem + loff) = ev[u];
-        }
+    for (int u = 0; u < NLE; ++u) {
+        long goff;
+        int loff;
+        tile_chunk(tid + u * NT, g.cbEt, goff, loff);
+        ev[u] = *(const bf16x8*)(Et + goff);
     }
-    __syncthreads();
+    __syncthreads();  // the operand stages are no longer read
 #pragma unroll
-    for (int i = 0; i < FM; ++i) {
-        // all LDS reads of a fragment row first (a write in between would serialise them)
-        bf16x4 e[FN][4];
+    for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-                e[j][q] = *(const bf16x4*)(smem + (wm * WTM + i * 32 + (lane & 31)) * S +
-                                           (wn * WTN + j * 32 + q * 8 + hi * 4) * 2);
-        bf16x4 o[FN][4];
+            for (int q = 0; q < 4; ++q) {
+                bf16x4 t;
 #pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    o[j][q][r] = f2bf(rbf(g.s0 * bf2f(e[j][q][r])) + rbf(acc[i][j][q * 4 + r]));
-#pragma unroll
-        for (int j = 0; j < FN; ++j)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                *(bf16x4*)(smem + (wm * WTM + i * 32 + (lane & 31)) * S + (wn * WTN + j * 32 + q * 8 + hi * 4) * 2) =
-                    o[j][q];
-    }
+                for (int r = 0; r < 4; ++r) t[r] = f2bf(acc[i][j][q * 4 + r]);
+                *(bf16x4*)(smem + (wm * WTM + i * 32 + (lane & 31)) * S + (wn * WTN + j * 32 + q * 8 + hi * 4) * 2) = t;
+            }
     __syncthreads();
     bf16_t* C = g.C + tc.bidx * g.strideC;
 #pragma unroll
@@ -316,7 +275,11 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
         long goff;
         int loff;
         tile_chunk(tid + u * NT, g.cbC, goff, loff);
-        *(u32x4*)(C + goff) = *(const u32x4*)(smem + loff);
+        const bf16x8 t = *(const bf16x8*)(smem + loff);
+        bf16x8 o;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o[k] = f2bf(rbf(g.s0 * bf2f(ev[u][k])) + bf2f(t[k]));
+        *(bf16x8*)(C + goff) = o;
     }
 }
 
