@@ -191,3 +191,57 @@ def test_tensor_list_table_rejects_cpu_tensors():
     with pytest.raises(_abi.MuonHipError):
         TensorListTable([[torch.zeros(3)]])
     assert _abi.MULTI_CHUNK == 16384
+
+
+def test_argument_errors_are_reported_before_any_launch():
+    """Every entry point rejects what it cannot run with a negative code and a message, before it
+    touches the device (so this runs without one)."""
+    lib = _abi.lib()
+    EINVAL, ESHAPE = -1, -2
+    ws = 0x1000  # never dereferenced: every call below is rejected on its arguments
+    tbl = 0x2000
+    F32, BF16 = _abi.dtype_code(torch.float32), _abi.dtype_code(torch.bfloat16)
+
+    def rejected(rc, code, needle):
+        assert rc == code, (rc, lib.muon_hip_last_error())
+        assert needle in lib.muon_hip_last_error().decode(), lib.muon_hip_last_error()
+
+    rejected(lib.muon_hip_momentum_norm(tbl, tbl, F32, F32, None, 8, 8, 1, 0.95, 1, 0, None), EINVAL, "workspace is null")
+    rejected(lib.muon_hip_momentum_norm(tbl, tbl, F32, F32, ws + 8, 8, 8, 1, 0.95, 1, 0, None), EINVAL, "256-byte aligned")
+    rejected(lib.muon_hip_momentum_norm(None, tbl, F32, F32, ws, 8, 8, 1, 0.95, 1, 0, None), EINVAL, "pointer table")
+    rejected(lib.muon_hip_momentum_norm(tbl, tbl, F32, BF16, ws, 8, 8, 1, 0.95, 1, 0, None), EINVAL, "dtypes")
+    rejected(lib.muon_hip_momentum_norm(tbl, tbl, F32, F32, ws, 8, 8, 70000, 0.95, 1, 0, None), ESHAPE, "65535")
+    rejected(lib.muon_hip_cast_norm(None, F32, ws, 8, 8, 1, None), EINVAL, "bad input")
+    rejected(lib.muon_hip_cast_norm(tbl, 7, ws, 8, 8, 1, None), EINVAL, "bad input")
+    rejected(lib.muon_hip_ns_grouped(ws, 8, 8, 1, -1, 1.0, 1.0, 1.0, None), EINVAL, "steps")
+    rejected(lib.muon_hip_ns_grouped(ws, 0, 8, 1, 5, 1.0, 1.0, 1.0, None), EINVAL, "positive")
+    rejected(lib.muon_hip_apply_update(None, F32, ws, 8, 8, 1, 5, 1.0, 0.02, 0.0, None), EINVAL, "bad pointer table")
+    rejected(lib.muon_hip_apply_update(tbl, 9, ws, 8, 8, 1, 5, 1.0, 0.02, 0.0, None), EINVAL, "dtype")
+    rejected(lib.muon_hip_ns_output(ws, 8, 8, 1, 5, None, None), EINVAL, "output pointer")
+    rejected(lib.muon_hip_step_grouped(tbl, tbl, tbl, F32, F32, F32, None, 8, 8, 1, 0.02, 0.0, 0.95, 1, 5, 1.0,
+                                       3.4445, -4.775, 2.0315, 0, None), EINVAL, "workspace is null")
+    assert lib.muon_hip_blocked_elems(256, 48) == 0 and b"multiple of 32" in lib.muon_hip_last_error()
+    assert lib.muon_hip_blocked_elems(300, 64) == 2 * 2 * 8192
+    rejected(lib.muon_hip_pack_bf16(None, 0, 64, 8, 64, tbl, 256, 64, 1, None), EINVAL, "null tensor")
+    rejected(lib.muon_hip_pack_bf16(tbl, 0, 32, 8, 64, tbl, 256, 64, 1, None), ESHAPE, "pack")
+    rejected(lib.muon_hip_unpack_bf16(tbl, 256, 48, tbl, 0, 64, 8, 48, 1, None), ESHAPE, "unpack")
+    rejected(lib.muon_hip_syrk_bf16(tbl, tbl, 256, 300, 1, _abi.CFG_AUTO, None), ESHAPE, "multiples")
+    rejected(lib.muon_hip_syrk_bf16(tbl, tbl, 512, 512, 1, 17, None), EINVAL, "unknown GEMM configuration")
+    rejected(lib.muon_hip_syrk_bf16(None, tbl, 512, 512, 1, _abi.CFG_AUTO, None), EINVAL, "null operand")
+    rejected(lib.muon_hip_sympoly_bf16(tbl, tbl, 512, 1, 1.0, 1.0, _abi.CFG_AUTO, None), EINVAL, "aliased")
+    rejected(lib.muon_hip_bx_axpy_bf16(tbl, tbl + 64, tbl + 64, 512, 512, 1, 1.0, _abi.CFG_AUTO, None), EINVAL, "alias")
+    rejected(lib.muon_hip_bx_axpy_bf16(tbl, tbl + 64, tbl + 128, 512, 640, 1, 1.0, _abi.CFG_256_PINGPONG, None),
+             ESHAPE, "multiples")
+    rejected(lib.muon_hip_adamw(None, tbl, tbl, tbl, F32, 4, 1, 1e-3, 0.9, 0.95, 1e-8, 0.0, None), EINVAL, "null tensor")
+    rejected(lib.muon_hip_adamw(tbl, tbl, tbl, tbl, F32, 4, 0, 1e-3, 0.9, 0.95, 1e-8, 0.0, None), EINVAL, "step")
+    assert lib.muon_hip_adamw(tbl, tbl, tbl, tbl, F32, 0, 1, 1e-3, 0.9, 0.95, 1e-8, 0.0, None) == 0  # empty tensor
+    rejected(lib.muon_hip_adamw_multi(tbl, tbl, tbl, tbl, tbl, tbl, tbl, tbl, 0, 1, F32, 1e-3, 0.9, 0.95, 1e-8, 0.0,
+                                      None), EINVAL, "at least one tensor")
+    rejected(lib.muon_hip_adamw_multi(tbl, tbl, tbl, tbl, tbl, tbl, None, tbl, 1, 1, F32, 1e-3, 0.9, 0.95, 1e-8, 0.0,
+                                      None), EINVAL, "null table")
+    rejected(lib.muon_hip_grad_norms(tbl, tbl, None, 1, 1, F32, tbl, tbl, None), EINVAL, "null tensor-list")
+    rejected(lib.muon_hip_grad_norms(tbl, tbl, tbl, 1, 1, F32, None, tbl, None), EINVAL, "null output")
+    rejected(lib.muon_hip_total_norm(tbl, 0, F32, tbl, tbl, None), EINVAL, "empty list")
+    rejected(lib.muon_hip_clip_scale(tbl, tbl, tbl, 1, 1, F32, None, F32, 1.0, None), EINVAL, "null total")
+    rejected(lib.muon_hip_clip_scale(tbl, tbl, tbl, 1, 1 << 31, F32, tbl, F32, 1.0, None), ESHAPE, "chunks exceed")
+    rejected(lib.muon_hip_timing_read(99, None, None), EINVAL, "kernel id")
