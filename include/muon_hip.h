@@ -88,6 +88,12 @@ int muon_hip_momentum_norm(const void* const* g_ptrs, const void* const* m_ptrs,
  * G is a dense [batch][rows][cols] tensor; workspace.U <- bf16(G) plus the partial sums. */
 int muon_hip_cast_norm(const void* G, int g_dtype, void* workspace, int rows, int cols, int batch, void* stream);
 
+/* The normalisation of fast_newtonschulz on its own, muon_utils.py:139-146, on what the first stage left in
+ * the workspace:  d = bf16(bf16(||U||_F) + 1e-7) from the partial sums (fixed order);  X <- bf16(U / d), written
+ * in the blocked operand layout, transposed when rows > cols (:139-140).  muon_hip_ns_grouped starts with it;
+ * muon_hip_ns_output(steps = 0) returns the normalised matrix. */
+int muon_hip_normalize(void* workspace, int rows, int cols, int batch, void* stream);
+
 /* fast_newtonschulz, muon_utils.py:139-156, on what the first stage left in the workspace:
  * normalise by bf16(bf16(||X||_F) + 1e-7), then `steps` iterations of
  *   A = X Xt; B = b A + c A A; X = a X + B X

@@ -32,6 +32,7 @@ SIGNATURES = {
     "muon_hip_momentum_norm": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int, c_double,
                                        c_int, c_int, c_void_p]),
     "muon_hip_cast_norm": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "muon_hip_normalize": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p]),
     "muon_hip_ns_grouped": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_double, c_double, c_double, c_void_p]),
     "muon_hip_apply_update": (c_int, [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_double, c_double,
                                       c_double, c_void_p]),

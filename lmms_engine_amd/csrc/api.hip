@@ -280,23 +280,29 @@ int muon_hip_cast_norm(const void* G, int g_dtype, void* workspace, int rows, in
     return e == hipSuccess ? 0 : hip_fail(e, "cast_norm launch");
 }
 
+int muon_hip_normalize(void* workspace, int rows, int cols, int batch, void* stream) {
+    Plan p;
+    if (int rc = make_plan(rows, cols, batch, p)) return rc;
+    if (int rc = check_ws(workspace)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_NORMALIZE, s);
+    hipError_t e = launch_normalize(wsp(workspace, p.offX[1]), p.strideU, (const float*)((char*)workspace + p.offParts),
+                                    p.nparts, (float*)((char*)workspace + p.offDenom), wsp(workspace, p.offX[0]),
+                                    p.strideX, rows, cols, p.Mp, p.Kp, batch, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "normalize launch");
+}
+
 int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int steps, double a, double b, double c,
                         void* stream) {
     Plan p;
     if (int rc = make_plan(rows, cols, batch, p)) return rc;
     if (int rc = check_ws(workspace)) return rc;
     if (steps < 0) return fail(MUON_HIP_EINVAL, "steps must be >= 0");
+    if (int rc = muon_hip_normalize(workspace, rows, cols, batch, stream)) return rc;
     hipStream_t s = (hipStream_t)stream;
     bf16_t* X[2] = {wsp(workspace, p.offX[0]), wsp(workspace, p.offX[1])};
     bf16_t* A = wsp(workspace, p.offA);
     bf16_t* B = wsp(workspace, p.offB);
-    {
-        Timed t(MUON_HIP_K_NORMALIZE, s);
-        hipError_t e = launch_normalize(X[1], p.strideU, (const float*)((char*)workspace + p.offParts), p.nparts,
-                                        (float*)((char*)workspace + p.offDenom), X[0], p.strideX, rows, cols, p.Mp, p.Kp,
-                                        batch, s);
-        if (e != hipSuccess) return hip_fail(e, "normalize launch");
-    }
     int cur = 0;
     for (int it = 0; it < steps; ++it) {
         if (int rc = do_syrk(pick_cfg(p.M, EPI_SYRK, p.Kp), X[cur], A, p.Mp, p.Kp, batch, s)) return rc;

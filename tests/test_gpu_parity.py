@@ -259,6 +259,35 @@ def test_newton_schulz_batched_matches_single_bitwise(env):
     assert torch.equal(stacked, mu.fast_newtonschulz(G, 5)), "run-to-run determinism"
 
 
+@pytest.mark.parametrize("rows,cols,batch", [(96, 200, 1), (200, 96, 2), (33, 47, 1), (512, 1024, 1)])
+def test_normalize_stage_on_its_own(env, rows, cols, batch):
+    """muon_hip_normalize after the first stage: X = bf(bf(G) / bf(bf(||bf(G)||_F) + 1e-7)) element for element
+    (muon_utils.py:138-146), the same through muon_hip_ns_grouped with no iterations, zero stays zero."""
+    print(f"normalize rows={rows} cols={cols} batch={batch}", flush=True)
+    lib, abi, dev = env["lib"], env["abi"], env["dev"]
+    G = torch.randn(batch, rows, cols, generator=torch.Generator().manual_seed(rows + cols + batch))
+    G[-1, 0, :5] = 0.0
+    X = G.bfloat16()
+    d = (X.float().pow(2).sum(dim=(-2, -1), keepdim=True).sqrt().bfloat16() + 1e-7).bfloat16()  # bf16 norm, bf16 add
+    ref = (X / d).bfloat16()
+    assert torch.equal(ref, (X / (X.norm(dim=(-2, -1), keepdim=True) + 1e-7))), "the literal torch expression"
+    Gd = G.to(dev)
+    ws = torch.empty(abi.workspace_bytes(rows, cols, batch), dtype=torch.uint8, device=dev)
+    out = [torch.full((batch, rows, cols), float("nan"), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+    for o, via_ns in zip(out, (False, True)):
+        abi.check(lib.muon_hip_cast_norm(Gd.data_ptr(), abi.dtype_code(Gd.dtype), ws.data_ptr(), rows, cols, batch, 0))
+        if via_ns:
+            abi.check(lib.muon_hip_ns_grouped(ws.data_ptr(), rows, cols, batch, 0, 3.4445, -4.775, 2.0315, 0))
+        else:
+            abi.check(lib.muon_hip_normalize(ws.data_ptr(), rows, cols, batch, 0))
+        abi.check(lib.muon_hip_ns_output(ws.data_ptr(), rows, cols, batch, 0, o.data_ptr(), 0))
+    torch.cuda.synchronize()
+    assert torch.equal(out[0], out[1])
+    # the device sums the squares in another order than torch, so for an unlucky sum the bf16 norm lands on the
+    # neighbouring value and every element moves by up to one part in 256; otherwise the result is exact
+    assert torch.equal(out[0].cpu(), ref) or rel_fro(out[0], ref) < 4.5e-3
+
+
 @pytest.mark.parametrize("gdt,mdt", [(torch.float32, torch.float32), (torch.bfloat16, torch.float32),
                                      (torch.bfloat16, torch.bfloat16)])
 @pytest.mark.parametrize("nesterov", [True, False])
