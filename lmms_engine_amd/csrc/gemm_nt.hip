@@ -112,8 +112,10 @@ __device__ __forceinline__ long panel_offset(int row0, int cb) {
 // into registers before the accumulators were written, and puts the sums back), while rows of C
 // are gathered with ds_read_b64_tr_b16: in a group of 16 lanes, lane i receives element i%4 of the
 // 8-byte pieces addressed by lanes i/4, 4+i/4, 8+i/4, 12+i/4.
-// Diagonal tiles of the symmetric kernels write the full tile once: acc(i,j) and acc(j,i) are
-// sums of the same exact products in the same order.
+// Diagonal tiles of the symmetric kernels: only the 32x32 fragments on or above the diagonal need to be
+// computed; the Ct pass writes them as the lower half (and the diagonal fragments) of the tile, the gather
+// writes the upper half.  Inside a diagonal fragment acc(i,j) and acc(j,i) are sums of the same exact products
+// in the same order, so the result is symmetric bit for bit.
 template <int BM, int BN>
 constexpr int epilogue_bytes() { return BN * (BM * 2 + 16); }
 
@@ -123,7 +125,7 @@ __device__ __forceinline__ s16x4 lds_read_tr16(const unsigned char* p) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(lds_void_ptr)p);
 }
 
-template <int BM, int BN, int WGM, int WGN, int EPI>
+template <int BM, int BN, int WGM, int WGN, int EPI, bool MASKED>
 __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
                                          f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], unsigned char* smem) {
     constexpr int NT = WGM * WGN * 64;
@@ -139,11 +141,16 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
     // Et and Ct hold the tile as rows n0.. (BN of them) x columns m0.. (BM of them).  Chunk c of a
     // thread: 16 bytes j = c%8 of the 128-byte row piece of row n = (c/8)%BN in column block c/8/BN,
     // so that a wave touches 8 rows x 128 bytes = 1 KB of one block, contiguous in memory.
+    // The return value says whether the chunk is a computed one: in a diagonal tile of a MASKED caller (the
+    // ping-pong kernel, which skips the others) only the 32x32 fragments on or above the diagonal are, i.e. column
+    // block m/32 <= row block n/32 of Tt.  A caller that computes whole diagonal tiles writes them in the Ct pass.
     auto tile_chunk = [&](int c, int cb, long& goff, int& loff) {
         constexpr int CPB = BLK_COLS / 8;  // 16-byte chunks per row of a block
+        static_assert(BLK_COLS == 32, "a column block is one fragment wide");
         const int j = c % CPB, n = (c / CPB) % BN, cbk = (c / CPB) / BN;
         goff = panel_offset(n0, cb) + (long)((m0 >> BLK_SHIFT) + cbk) * BLK_ELEMS + n * BLK_COLS + j * 8;
         loff = n * S + (cbk * CPB + j) * 16;
+        return !MASKED || !diag || cbk <= (n >> 5);
     };
     // SYMPOLY: this thread's 16-byte pieces of the b.A term, in the layout of the Ct pass, go to registers
     // first, so that the loads are in flight while the accumulators are rounded into LDS
@@ -183,18 +190,18 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
         for (int u = 0; u < NLE; ++u) {
             long goff;
             int loff;
-            tile_chunk(tid + u * NT, g.cbCt, goff, loff);
+            const bool computed = tile_chunk(tid + u * NT, g.cbCt, goff, loff);
             bf16x8 t = *(const bf16x8*)(smem + loff);
             if (EPI == EPI_SYMPOLY) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k) t[k] = f2bf(rbf(g.s0 * bf2f(ev[u][k])) + bf2f(t[k]));
-                if (!diag) *(bf16x8*)(smem + loff) = t;
+                if (MASKED ? computed : !diag) *(bf16x8*)(smem + loff) = t;
             }
-            if (g.Ct) *(bf16x8*)(Ct + goff) = t;
+            if (g.Ct && computed) *(bf16x8*)(Ct + goff) = t;
         }
-        if (EPI == EPI_SYMPOLY && !diag) __syncthreads();
+        if (EPI == EPI_SYMPOLY && (MASKED || !diag)) __syncthreads();
     }
-    if (g.C && !diag) {
+    if (g.C && (MASKED || !diag)) {
         // lane j = 4r+s of a group addresses row n + 8s + r (then + 4), pieces m = 4c..4c+3: lane i = 4s+e
         // receives Tt[n+8s .. n+8s+7][4c+e], 16 bytes of row 4c+e of C.  The four groups of a wave sit
         // side by side along n (128 columns = two column blocks): 4 rows x 128 bytes per block and store.
@@ -212,7 +219,10 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
             const unsigned char* q = src + strip * 128 * S + c * 8;
             const s16x4 lo = lds_read_tr16(q), hi4 = lds_read_tr16(q + 4 * S);
             const s16x8 o = {lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
-            *(s16x8*)(dst + (long)strip * (128 / BLK_COLS) * BLK_ELEMS + c * 4 * BLK_COLS) = o;
+            // a diagonal tile: the pieces strictly above the diagonal fragments (row block c/8 < column block);
+            // the Ct pass has written the rest
+            if (!diag || (c >> 3) < strip * 4 + grp)
+                *(s16x8*)(dst + (long)strip * (128 / BLK_COLS) * BLK_ELEMS + c * 4 * BLK_COLS) = o;
         }
     }
 }
@@ -454,7 +464,24 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     }
     WAIT_VM(0);  // the dummy loads of the last two tails must not land in the epilogue's tile
     if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN>(g, tc, acc, smem);
-    else epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    else epilogue<BM, BN, WGM, WGN, EPI, false>(g, tc, acc, smem);
+}
+
+// Fragments (i, j) of wave `wave` of a WGM x WGN wave grid that lie entirely below the diagonal of a diagonal tile.
+template <int WTM, int WTN, int FM, int FN, int WGN>
+constexpr unsigned pp_skip_mask(int wave) {
+    const int wm = wave / WGN, wn = wave % WGN;
+    unsigned m = 0;
+    for (int i = 0; i < FM; ++i)
+        for (int j = 0; j < FN; ++j)
+            if (wm * WTM + i * 32 >= wn * WTN + j * 32 + 32) m |= 1u << (i * FN + j);
+    return m;
+}
+template <int WTM, int WTN, int FM, int FN, int WGN>
+constexpr bool pp_first_with_mask(int wave) {
+    for (int w = 0; w < wave; ++w)
+        if (pp_skip_mask<WTM, WTN, FM, FN, WGN>(w) == pp_skip_mask<WTM, WTN, FM, FN, WGN>(wave)) return false;
+    return true;
 }
 
 // ---- kernel 2: eight waves in two groups that alternate between memory and MFMA phases --------
@@ -540,6 +567,10 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+    // Diagonal tile of a symmetric product: a fragment of a wave that lies entirely below the diagonal is the
+    // mirror image of one another wave computes, and the epilogue does not read it.  Bit i*FN+j of a wave's mask:
+    // skip that fragment's MFMAs (and the fragment reads nobody needs).
+    const bool diag = EPI != EPI_BX && tc.ti == tc.tj;
     const int sw = (lane >> 2) & 3, hi = lane >> 5;
     const int a_off = (wm * WTM + (lane & 31)) * ROWB;
     const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROWB;
@@ -567,17 +598,27 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
                               : smem + half * 2 * STAGE + b_off + co;
         }
     }
-    auto body = [&](int kt, auto stage_c) {
+    auto body = [&](int kt, auto stage_c, auto mask_c) {
         constexpr int SIDX = decltype(stage_c)::value;
+        constexpr unsigned MASK = decltype(mask_c)::value;
+        auto kept = [](int i, int j) { return !((MASK >> (i * FN + j)) & 1); };
         // ---- M(kt)
         bf16x8 fa[2][FM], fb[2][FN];
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
-                fa[ks][i] = *(const bf16x8*)(ra[ks][SIDX >> 1] + (SIDX & 1) * STAGE + i * 32 * ROWB);
+            for (int i = 0; i < FM; ++i) {
+                bool used = false;
+#pragma unroll
+                for (int j = 0; j < FN; ++j) used |= kept(i, j);
+                if (used) fa[ks][i] = *(const bf16x8*)(ra[ks][SIDX >> 1] + (SIDX & 1) * STAGE + i * 32 * ROWB);
+            }
 #pragma unroll
             for (int j = 0; j < FN; ++j) {
+                bool used = false;
+#pragma unroll
+                for (int i = 0; i < FM; ++i) used |= kept(i, j);
+                if (!used) continue;
                 if (QT) fb[ks][j] = lds_read_qt(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 2048);
                 else fb[ks][j] = *(const bf16x8*)(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 32 * ROWB);
             }
@@ -599,7 +640,7 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
                 for (int j = 0; j < FN; ++j) {
                     if (QT)  // operands swapped: a lane then holds 4 consecutive columns of one row of the tile
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
-                    else
+                    else if (kept(i, j))
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
                 }
         __builtin_amdgcn_sched_barrier(0);
@@ -609,16 +650,39 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
         __builtin_amdgcn_sched_barrier(0);
     };
     // nk is a multiple of 4 (k extents are multiples of 128)
-    for (int kt = 0; kt < nk; kt += 4) {
-        body(kt, std::integral_constant<int, 0>{});
-        body(kt + 1, std::integral_constant<int, 1>{});
-        body(kt + 2, std::integral_constant<int, 2>{});
-        body(kt + 3, std::integral_constant<int, 3>{});
+    auto k_loop = [&](auto mask_c) {
+        for (int kt = 0; kt < nk; kt += 4) {
+            body(kt, std::integral_constant<int, 0>{}, mask_c);
+            body(kt + 1, std::integral_constant<int, 1>{}, mask_c);
+            body(kt + 2, std::integral_constant<int, 2>{}, mask_c);
+            body(kt + 3, std::integral_constant<int, 3>{}, mask_c);
+        }
+    };
+    // One copy of the loop per distinct mask (the masks are compile-time facts of the wave grid), chosen once per
+    // tile: no test inside the loop.  Tiles off the diagonal, nearly all, take the first.
+    if (!diag) {
+        k_loop(std::integral_constant<unsigned, 0>{});
+    } else {
+        auto run_if_mine = [&](auto wave_c) {
+            constexpr int W = decltype(wave_c)::value;
+            constexpr unsigned M = pp_skip_mask<WTM, WTN, FM, FN, WGN>(W);
+            if constexpr (pp_first_with_mask<WTM, WTN, FM, FN, WGN>(W)) {
+                if (pp_skip_mask<WTM, WTN, FM, FN, WGN>(wave) == M) k_loop(std::integral_constant<unsigned, M>{});
+            }
+        };
+        run_if_mine(std::integral_constant<int, 0>{});
+        run_if_mine(std::integral_constant<int, 1>{});
+        run_if_mine(std::integral_constant<int, 2>{});
+        run_if_mine(std::integral_constant<int, 3>{});
+        run_if_mine(std::integral_constant<int, 4>{});
+        run_if_mine(std::integral_constant<int, 5>{});
+        run_if_mine(std::integral_constant<int, 6>{});
+        run_if_mine(std::integral_constant<int, 7>{});
     }
     if (!grp) __builtin_amdgcn_s_barrier();
     WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
     if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN>(g, tc, acc, smem);
-    else epilogue<BM, BN, WGM, WGN, EPI>(g, tc, acc, smem);
+    else epilogue<BM, BN, WGM, WGN, EPI, true>(g, tc, acc, smem);
 }
 
 template <int BM, int BN, int WGM, int WGN, int EPI>
