@@ -30,7 +30,7 @@ PEAK_HBM_GBS = 8000.0
 # rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over this script, each scaled by what the same counter
 # reads for the 1 GiB copy of --calibrate-copy (one FETCH_SIZE unit = 2 KiB, one WRITE_SIZE unit = 1 KiB).
 # A counter run cannot share a process with the event timing, so the figure is carried here.
-BX_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 24.099e9 + 3.473e9}
+BX_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 23.455e9 + 3.473e9}
 
 WORKLOADS = {
     "qwen3-8b": dict(layers=36, shapes=dict(q=(4096, 4096), k=(1024, 4096), v=(1024, 4096), o=(4096, 4096),
