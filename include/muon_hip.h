@@ -158,6 +158,21 @@ int muon_hip_bx_axpy_bf16(const void* B, const void* X, void* Xout, int Mp, int 
 int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int dtype, long n, int step, double lr,
                    double beta1, double beta2, double eps, double weight_decay, void* stream);
 
+/* adam_update on its own, muon_utils.py:178-183: exp_avg and exp_avg_sq move in place, the bias-corrected
+ * update exp_avg_c / (sqrt(exp_avg_sq_c) + eps) is written to `out` (n elements of `dtype`, may not alias). */
+int muon_hip_adam_update(const void* g, void* exp_avg, void* exp_avg_sq, void* out, int dtype, long n, int step,
+                         double beta1, double beta2, double eps, void* stream);
+
+/* apply_scaling on its own, muon_utils.py:167-175: x <- x * scale in place, one rounding in x's dtype. */
+int muon_hip_scale(void* x, int dtype, long n, double scale, void* stream);
+
+/* The decay and update lines on a dense update tensor, muon_utils.py:406-407 (the Muon branch of
+ * step_deepspeed, where DeepSpeed has already put the orthogonalised update into p.grad) and :324-325:
+ *   p <- p * (1 - lr*wd);  p <- p + (-lr) * u
+ * (p, u) dtypes: (f32, f32), (bf16, bf16), (f32, bf16). */
+int muon_hip_decay_update(void* p, int p_dtype, const void* u, int u_dtype, long n, double lr, double weight_decay,
+                          void* stream);
+
 /* ---- multi-tensor kernels ---------------------------------------------------------------
  * One launch walks a list of n tensors of one dtype.  The list is described by device arrays:
  * base pointers (`const void* const*`, n entries), element counts `numel` (n longs) and

@@ -3,6 +3,7 @@ from .muon_utils import (  # noqa: F401
     Muon,
     SingelDeviceWork,
     Work,
+    adam_update,
     apply_momentum,
     apply_scaling,
     fast_newtonschulz,
@@ -15,6 +16,7 @@ __all__ = [
     "Muon",
     "SingelDeviceWork",
     "Work",
+    "adam_update",
     "apply_momentum",
     "apply_scaling",
     "fast_newtonschulz",

@@ -48,6 +48,10 @@ SIGNATURES = {
     "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_int, c_void_p]),
     "muon_hip_adamw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_double,
                                c_double, c_double, c_double, c_void_p]),
+    "muon_hip_adam_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_double,
+                                     c_double, c_void_p]),
+    "muon_hip_scale": (c_int, [c_void_p, c_int, c_long, c_double, c_void_p]),
+    "muon_hip_decay_update": (c_int, [c_void_p, c_int, c_void_p, c_int, c_long, c_double, c_double, c_void_p]),
     "muon_hip_adamw_multi": (c_int, [c_void_p] * 8 + [c_int, c_long, c_int] + [c_double] * 5 + [c_void_p]),
     "muon_hip_grad_norms": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_void_p, c_void_p]),
     "muon_hip_total_norm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),

@@ -2,6 +2,7 @@
 // partitioning, the grouped launch sequence of one Muon step, and per-kernel event timing.
 #include <stdarg.h>
 #include <stdio.h>
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -14,7 +15,7 @@
 namespace {
 
 thread_local char g_err[512] = "";
-int g_forced_cfg = MUON_HIP_CFG_AUTO;
+std::atomic<int> g_forced_cfg{MUON_HIP_CFG_AUTO};  // benchmarking override, read once per call
 
 int fail(int code, const char* fmt, ...) {
     va_list ap;
@@ -34,7 +35,7 @@ struct EventPair {
     hipEvent_t start, stop;
 };
 std::mutex g_tmu;
-bool g_timing = false;
+std::atomic<bool> g_timing{false};
 std::vector<EventPair> g_events[MUON_HIP_K_COUNT];
 constexpr size_t kMaxEventsPerKernel = 1 << 16;
 
@@ -54,7 +55,7 @@ struct Timed {
     EventPair ev;
     bool on;
     Timed(int k, hipStream_t st) : kid(k), s(st), on(false) {
-        if (!g_timing) return;
+        if (!g_timing.load(std::memory_order_acquire)) return;
         std::lock_guard<std::mutex> lk(g_tmu);
         if (g_events[kid].size() >= kMaxEventsPerKernel) return;
         if (hipEventCreate(&ev.start) != hipSuccess) return;
@@ -88,7 +89,8 @@ bool use_tile256(int M) { return M % 256 == 0 && M >= 512; }
 // Configuration per kernel, from a sweep of every variant over the benchmark shapes: the ping-pong
 // kernel wherever 256-tiles fill the machine, 128-tiles for the symmetric products of small matrices.
 int pick_cfg(int M, int epi = EPI_BX, int kdim = 0) {
-    if (g_forced_cfg != MUON_HIP_CFG_AUTO) return g_forced_cfg;
+    const int forced = g_forced_cfg.load(std::memory_order_relaxed);
+    if (forced != MUON_HIP_CFG_AUTO) return forced;
     (void)kdim;
     if (!use_tile256(M)) return GEMM_CFG_128_PIPE;
     if (epi != EPI_BX && M <= 512) return GEMM_CFG_128_PIPE;
@@ -229,7 +231,7 @@ const char* muon_hip_last_error(void) { return g_err; }
 
 int muon_hip_set_gemm_config(int cfg) {
     if (cfg != MUON_HIP_CFG_AUTO && gemm_cfg_tile(cfg) == 0) return fail(MUON_HIP_EINVAL, "unknown GEMM configuration %d", cfg);
-    g_forced_cfg = cfg;
+    g_forced_cfg.store(cfg, std::memory_order_relaxed);
     return 0;
 }
 
@@ -415,6 +417,38 @@ int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int 
     return e == hipSuccess ? 0 : hip_fail(e, "adamw launch");
 }
 
+int muon_hip_adam_update(const void* g, void* exp_avg, void* exp_avg_sq, void* out, int dtype, long n, int step,
+                         double beta1, double beta2, double eps, void* stream) {
+    if (!g || !exp_avg || !exp_avg_sq || !out) return fail(MUON_HIP_EINVAL, "null tensor");
+    if (!dtype_ok(dtype) || n < 0 || step < 1) return fail(MUON_HIP_EINVAL, "bad dtype, size or step");
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_ADAMW, s);
+    hipError_t e = launch_adam_update(g, exp_avg, exp_avg_sq, out, dtype, n, step, beta1, beta2, eps, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "adam_update launch");
+}
+
+int muon_hip_scale(void* x, int dtype, long n, double scale, void* stream) {
+    if (!x) return fail(MUON_HIP_EINVAL, "null tensor");
+    if (!dtype_ok(dtype) || n < 0) return fail(MUON_HIP_EINVAL, "bad dtype or size");
+    if (n == 0) return 0;
+    hipError_t e = launch_scale(x, dtype, n, scale, (hipStream_t)stream);
+    return e == hipSuccess ? 0 : hip_fail(e, "scale launch");
+}
+
+int muon_hip_decay_update(void* p, int p_dtype, const void* u, int u_dtype, long n, double lr, double weight_decay,
+                          void* stream) {
+    if (!p || !u) return fail(MUON_HIP_EINVAL, "null tensor");
+    if (!dtype_ok(p_dtype) || !dtype_ok(u_dtype) || n < 0) return fail(MUON_HIP_EINVAL, "bad dtype or size");
+    if (p_dtype == MUON_HIP_BF16 && u_dtype == MUON_HIP_F32)
+        return fail(MUON_HIP_EINVAL, "an fp32 update for a bf16 parameter is not supported");
+    if (n == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_UPDATE, s);
+    hipError_t e = launch_decay_update(p, p_dtype, u, u_dtype, n, lr, weight_decay, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "decay_update launch");
+}
+
 namespace {
 int check_list(const void* ptrs, const long* numel, const long* chunk_start, int n, long chunks, int dtype) {
     if (!ptrs || !numel || !chunk_start) return fail(MUON_HIP_EINVAL, "null tensor-list array");
@@ -471,7 +505,7 @@ int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long
 int muon_hip_timing_enable(int on) {
     std::lock_guard<std::mutex> lk(g_tmu);
     clear_events();
-    g_timing = on != 0;
+    g_timing.store(on != 0, std::memory_order_release);
     return 0;
 }
 

@@ -22,3 +22,8 @@ hipError_t launch_pack(const bf16_t* src, long strideSrc, int ld, int rows, int 
                        int rows_p, int cols_p, int batch, hipStream_t stream);
 hipError_t launch_adamw(void* p, const void* g, void* e1, void* e2, int dtype, long n, int step, double lr,
                         double b1, double b2, double eps, double wd, hipStream_t stream);
+hipError_t launch_adam_update(const void* g, void* e1, void* e2, void* out, int dtype, long n, int step, double b1,
+                              double b2, double eps, hipStream_t stream);
+hipError_t launch_scale(void* x, int dtype, long n, double s, hipStream_t stream);
+hipError_t launch_decay_update(void* p, int p_dtype, const void* u, int u_dtype, long n, double lr, double wd,
+                               hipStream_t stream);

@@ -156,7 +156,8 @@ momentum_norm_kernel(const void* const* g_ptrs, const void* const* m_ptrs, bf16_
 }
 
 // Sum of squares of an existing bf16 (or fp32, rounded to bf16 first) matrix: the
-// Frobenius stage of fast_newtonschulz when it is called on its own.
+// Frobenius stage of fast_newtonschulz when it is called on its own.  16-byte accesses when the
+// matrix base and the batch strides allow it, scalars otherwise and for the last few elements.
 template <typename GT>
 __global__ void __launch_bounds__(256)
 cast_norm_kernel(const GT* G, long strideG, bf16_t* U, long strideU, float* partials, long n) {
@@ -165,7 +166,21 @@ cast_norm_kernel(const GT* G, long strideG, bf16_t* U, long strideU, float* part
     const GT* g = G + b * strideG;
     bf16_t* u = U + b * strideU;
     float ss = 0.f;
-    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+    const bool vec = ((((uintptr_t)g) | ((uintptr_t)u)) & 15) == 0;
+    const long n8 = vec ? n / 8 : 0;
+    for (long i8 = (long)blockIdx.x * 256 + threadIdx.x; i8 < n8; i8 += (long)gridDim.x * 256) {
+        float v[8];
+        Ld<GT>::load8(g + i8 * 8, v);
+        bf16x8 ub;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            ub[i] = f2bf(v[i]);
+            const float uu = bf2f(ub[i]);
+            ss = fmaf(uu, uu, ss);
+        }
+        *(bf16x8*)(u + i8 * 8) = ub;
+    }
+    for (long i = n8 * 8 + (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
         const float uu = rbf(Ld<GT>::load(g + i));
         u[i] = f2bf(uu);
         ss = fmaf(uu, uu, ss);
@@ -346,16 +361,48 @@ apply_update_t_kernel(const void* const* p_ptrs, const bf16_t* O, long strideO, 
 }
 
 // A blocked matrix, or its transpose, into a dense row-major bf16 tensor (row pitch ld): the NS output of
-// fast_newtonschulz called alone, and the result of a single GEMM.
+// fast_newtonschulz called alone, and the result of a single GEMM.  One workgroup moves a tile of 64 output rows
+// x 128 output columns: straight (16-byte pieces of rows of the blocked image) or, for the transpose, from 128
+// rows x 64 columns of the blocked image through LDS.  Output rows leave as 16-byte vectors when the row pitch
+// and the base allow it.
 __global__ void __launch_bounds__(256)
 unpack_kernel(bf16_t* out, long strideOut, int ld, const bf16_t* O, long strideO, int cbo, int rows, int cols,
               int transposed) {
+    constexpr int TR = 64, TC = 128, PITCH = TR + 8;
+    __shared__ __align__(16) bf16_t tile[TC][PITCH];  // transposed case: tile[c][r]
     const int b = blockIdx.y;
-    const long n = (long)rows * cols;
-    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
-        const long r = i / cols;
-        const int c = (int)(i - r * cols);
-        out[b * strideOut + r * ld + c] = O[b * strideO + (transposed ? blocked_offset(c, r, cbo) : blocked_offset(r, c, cbo))];
+    bf16_t* dst = out + b * strideOut;
+    const bf16_t* o = O + b * strideO;
+    const int tiles_c = (cols + TC - 1) / TC;
+    const int r0 = (blockIdx.x / tiles_c) * TR, c0 = (blockIdx.x % tiles_c) * TC;
+    const bool vec = (ld % 8 == 0) && ((((uintptr_t)dst) & 15) == 0);
+    const int pr = threadIdx.x >> 4, pc = (threadIdx.x & 15) * 8;  // 16 rows x 16 chunks per pass
+    if (transposed) {
+        // image rows c0..c0+127, columns r0..r0+63; the blocked image is padded to whole 128-tiles in both
+        // directions, so these reads stay inside it
+        const int xr = threadIdx.x >> 3, xc = (threadIdx.x & 7) * 8;
+#pragma unroll
+        for (int h = 0; h < 4; ++h)
+            *(bf16x8*)(&tile[xr + h * 32][xc]) = *(const bf16x8*)(o + blocked_offset(c0 + xr + h * 32, r0 + xc, cbo));
+        __syncthreads();
+    }
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+        const int r = r0 + pr + h * 16, c = c0 + pc;
+        if (r >= rows || c >= cols) continue;
+        bf16x8 v;
+        if (transposed) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = tile[pc + i][pr + h * 16];
+        } else {
+            v = *(const bf16x8*)(o + blocked_offset(r, c, cbo));  // columns c..c+7 lie in one block row (c % 8 == 0)
+        }
+        bf16_t* d = dst + (long)r * ld + c;
+        if (vec && c + 8 <= cols) {
+            *(bf16x8*)d = v;
+        } else {
+            for (int i = 0; i < 8 && c + i < cols; ++i) d[i] = v[i];
+        }
     }
 }
 
@@ -371,34 +418,108 @@ pack_kernel(const bf16_t* src, long strideSrc, int ld, int rows, int cols, bf16_
         const long r = i / (cols_p / 8);
         const int c = (int)(i - r * (cols_p / 8)) * 8;
         bf16x8 v;
+        const bf16_t* sp = src + b * strideSrc + r * ld + c;
+        if (r < rows && c + 8 <= cols && ((((uintptr_t)sp) & 15) == 0)) {
+            v = *(const bf16x8*)sp;
+        } else {
 #pragma unroll
-        for (int k = 0; k < 8; ++k) v[k] = (r < rows && c + k < cols) ? src[b * strideSrc + r * ld + c + k] : (bf16_t)0.f;
+            for (int k = 0; k < 8; ++k) v[k] = (r < rows && c + k < cols) ? sp[k] : (bf16_t)0.f;
+        }
         *(bf16x8*)(dst + b * strideDst + blocked_offset(r, c, cb)) = v;
     }
 }
 
 struct AdamMath {
-    float w1, w1m1, w2, w2m1, c1, c2, eps, decay, alpha;
+    float w1, w1m1, w2, w2m1, r1, r2, eps, decay, alpha;  // r1, r2: reciprocals of the bias corrections
     bool small1, small2;
 };
+
+// adam_update (muon_utils.py:178-183) for one element, every in-place op rounded in the tensor dtype.  A tensor
+// divided by a python scalar is evaluated on a GPU as a multiplication by the scalar's fp32 reciprocal.
+template <typename T>
+__device__ __forceinline__ float adam_moments(float gi, float& e1, float& e2, const AdamMath& am) {
+    const float a = Ld<T>::rnd(lerp_aten(e1, gi, am.w1, am.w1m1, am.small1));
+    const float g2 = Ld<T>::rnd(gi * gi);
+    const float bb = Ld<T>::rnd(lerp_aten(e2, g2, am.w2, am.w2m1, am.small2));
+    e1 = a;
+    e2 = bb;
+    const float ac = Ld<T>::rnd(a * am.r1);
+    const float bc = Ld<T>::rnd(bb * am.r2);
+    const float den = Ld<T>::rnd(Ld<T>::rnd(__fsqrt_rn(bc)) + am.eps);
+    return Ld<T>::rnd(__fdiv_rn(ac, den));
+}
 
 template <typename T>
 __global__ void __launch_bounds__(256)
 adamw_kernel(T* p, const T* g, T* e1, T* e2, long n, AdamMath am) {
     for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
-        const float gi = Ld<T>::load(g + i);
-        const float a = Ld<T>::rnd(lerp_aten(Ld<T>::load(e1 + i), gi, am.w1, am.w1m1, am.small1));
-        const float g2 = Ld<T>::rnd(gi * gi);
-        const float bb = Ld<T>::rnd(lerp_aten(Ld<T>::load(e2 + i), g2, am.w2, am.w2m1, am.small2));
+        float a = Ld<T>::load(e1 + i), bb = Ld<T>::load(e2 + i);
+        const float upd = adam_moments<T>(Ld<T>::load(g + i), a, bb, am);
         Ld<T>::store(e1 + i, a);
         Ld<T>::store(e2 + i, bb);
-        const float ac = Ld<T>::rnd(__fdiv_rn(a, am.c1));
-        const float bc = Ld<T>::rnd(__fdiv_rn(bb, am.c2));
-        const float den = Ld<T>::rnd(Ld<T>::rnd(__fsqrt_rn(bc)) + am.eps);
-        const float upd = Ld<T>::rnd(__fdiv_rn(ac, den));
         const float pd = Ld<T>::rnd(Ld<T>::load(p + i) * am.decay);
         Ld<T>::store(p + i, fmaf(am.alpha, upd, pd));
     }
+}
+
+// adam_update on its own: the moments move in place, the update goes to `out`.
+template <typename T>
+__global__ void __launch_bounds__(256)
+adam_update_kernel(const T* g, T* e1, T* e2, T* out, long n, AdamMath am) {
+    const bool vec = ((((uintptr_t)g) | ((uintptr_t)e1) | ((uintptr_t)e2) | ((uintptr_t)out)) & 15) == 0;
+    const long n8 = vec ? n / 8 : 0;
+    for (long i8 = (long)blockIdx.x * 256 + threadIdx.x; i8 < n8; i8 += (long)gridDim.x * 256) {
+        float gv[8], av[8], bv[8], uv[8];
+        Ld<T>::load8(g + i8 * 8, gv);
+        Ld<T>::load8(e1 + i8 * 8, av);
+        Ld<T>::load8(e2 + i8 * 8, bv);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) uv[k] = adam_moments<T>(gv[k], av[k], bv[k], am);
+        Ld<T>::store8(e1 + i8 * 8, av);
+        Ld<T>::store8(e2 + i8 * 8, bv);
+        Ld<T>::store8(out + i8 * 8, uv);
+    }
+    for (long i = n8 * 8 + (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+        float a = Ld<T>::load(e1 + i), bb = Ld<T>::load(e2 + i);
+        const float upd = adam_moments<T>(Ld<T>::load(g + i), a, bb, am);
+        Ld<T>::store(e1 + i, a);
+        Ld<T>::store(e2 + i, bb);
+        Ld<T>::store(out + i, upd);
+    }
+}
+
+// x <- rnd(x * s): apply_scaling on its own (muon_utils.py:167-175).
+template <typename T>
+__global__ void __launch_bounds__(256) scale_kernel(T* x, long n, float s) {
+    const bool vec = (((uintptr_t)x) & 15) == 0;
+    const long n8 = vec ? n / 8 : 0;
+    for (long i8 = (long)blockIdx.x * 256 + threadIdx.x; i8 < n8; i8 += (long)gridDim.x * 256) {
+        float v[8];
+        Ld<T>::load8(x + i8 * 8, v);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] *= s;
+        Ld<T>::store8(x + i8 * 8, v);
+    }
+    for (long i = n8 * 8 + (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+        Ld<T>::store(x + i, Ld<T>::load(x + i) * s);
+}
+
+// p <- rnd(p * decay); p <- rnd(p + alpha * u): the decay and update lines on a dense update tensor u
+// (muon_utils.py:406-407, the Muon branch of step_deepspeed, and :324-325).
+template <typename PT, typename UT>
+__global__ void __launch_bounds__(256) decay_update_kernel(PT* p, const UT* u, long n, float decay, float alpha) {
+    const bool vec = ((((uintptr_t)p) | ((uintptr_t)u)) & 15) == 0;
+    const long n8 = vec ? n / 8 : 0;
+    for (long i8 = (long)blockIdx.x * 256 + threadIdx.x; i8 < n8; i8 += (long)gridDim.x * 256) {
+        float pv[8], uv[8];
+        Ld<PT>::load8(p + i8 * 8, pv);
+        Ld<UT>::load8(u + i8 * 8, uv);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) pv[k] = fmaf(alpha, uv[k], Ld<PT>::rnd(pv[k] * decay));
+        Ld<PT>::store8(p + i8 * 8, pv);
+    }
+    for (long i = n8 * 8 + (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256)
+        Ld<PT>::store(p + i, fmaf(alpha, Ld<UT>::load(u + i), Ld<PT>::rnd(Ld<PT>::load(p + i) * decay)));
 }
 
 inline int blocks_for(long n, int per_block, int cap) {
@@ -496,7 +617,7 @@ hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf1
 
 hipError_t launch_unpack(bf16_t* out, long strideOut, int ld, const bf16_t* O, long strideO, int cbo, int rows,
                          int cols, bool transposed, int batch, hipStream_t stream) {
-    dim3 grid(blocks_for((long)rows * cols, 256 * 8, 2048), batch), block(256);
+    dim3 grid(((rows + 63) / 64) * ((cols + 127) / 128), batch), block(256);
     hipLaunchKernelGGL(unpack_kernel, grid, block, 0, stream, out, strideOut, ld, O, strideO, cbo, rows, cols,
                        transposed ? 1 : 0);
     return hipGetLastError();
@@ -509,16 +630,23 @@ hipError_t launch_pack(const bf16_t* src, long strideSrc, int ld, int rows, int 
     return hipGetLastError();
 }
 
-hipError_t launch_adamw(void* p, const void* g, void* e1, void* e2, int dtype, long n, int step, double lr,
-                        double b1, double b2, double eps, double wd, hipStream_t stream) {
+namespace {
+AdamMath adam_math(int step, double lr, double b1, double b2, double eps, double wd) {
     AdamMath am;
     lerp_consts(1.0 - b1, am.w1, am.w1m1, am.small1);
     lerp_consts(1.0 - b2, am.w2, am.w2m1, am.small2);
-    am.c1 = (float)(1.0 - pow(b1, (double)step));
-    am.c2 = (float)(1.0 - pow(b2, (double)step));
+    am.r1 = 1.0f / (float)(1.0 - pow(b1, (double)step));
+    am.r2 = 1.0f / (float)(1.0 - pow(b2, (double)step));
     am.eps = (float)eps;
     am.decay = (float)(1.0 - lr * wd);
     am.alpha = (float)(-lr);
+    return am;
+}
+}  // namespace
+
+hipError_t launch_adamw(void* p, const void* g, void* e1, void* e2, int dtype, long n, int step, double lr,
+                        double b1, double b2, double eps, double wd, hipStream_t stream) {
+    const AdamMath am = adam_math(step, lr, b1, b2, eps, wd);
     dim3 grid(blocks_for(n, 256 * 4, 8192)), block(256);
     if (dtype == MUON_HIP_F32)
         hipLaunchKernelGGL((adamw_kernel<float>), grid, block, 0, stream, (float*)p, (const float*)g, (float*)e1,
@@ -526,6 +654,44 @@ hipError_t launch_adamw(void* p, const void* g, void* e1, void* e2, int dtype, l
     else if (dtype == MUON_HIP_BF16)
         hipLaunchKernelGGL((adamw_kernel<bf16_t>), grid, block, 0, stream, (bf16_t*)p, (const bf16_t*)g, (bf16_t*)e1,
                            (bf16_t*)e2, n, am);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_adam_update(const void* g, void* e1, void* e2, void* out, int dtype, long n, int step, double b1,
+                              double b2, double eps, hipStream_t stream) {
+    const AdamMath am = adam_math(step, 0.0, b1, b2, eps, 0.0);
+    dim3 grid(blocks_for(n, 256 * 8 * 2, 8192)), block(256);
+    if (dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((adam_update_kernel<float>), grid, block, 0, stream, (const float*)g, (float*)e1, (float*)e2,
+                           (float*)out, n, am);
+    else if (dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((adam_update_kernel<bf16_t>), grid, block, 0, stream, (const bf16_t*)g, (bf16_t*)e1,
+                           (bf16_t*)e2, (bf16_t*)out, n, am);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_scale(void* x, int dtype, long n, double s, hipStream_t stream) {
+    dim3 grid(blocks_for(n, 256 * 8 * 2, 8192)), block(256);
+    if (dtype == MUON_HIP_F32) hipLaunchKernelGGL((scale_kernel<float>), grid, block, 0, stream, (float*)x, n, (float)s);
+    else if (dtype == MUON_HIP_BF16) hipLaunchKernelGGL((scale_kernel<bf16_t>), grid, block, 0, stream, (bf16_t*)x, n, (float)s);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
+hipError_t launch_decay_update(void* p, int p_dtype, const void* u, int u_dtype, long n, double lr, double wd,
+                               hipStream_t stream) {
+    const float decay = (float)(1.0 - lr * wd), alpha = (float)(-lr);
+    dim3 grid(blocks_for(n, 256 * 8 * 2, 8192)), block(256);
+    if (p_dtype == MUON_HIP_F32 && u_dtype == MUON_HIP_F32)
+        hipLaunchKernelGGL((decay_update_kernel<float, float>), grid, block, 0, stream, (float*)p, (const float*)u, n, decay, alpha);
+    else if (p_dtype == MUON_HIP_F32 && u_dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((decay_update_kernel<float, bf16_t>), grid, block, 0, stream, (float*)p, (const bf16_t*)u, n, decay, alpha);
+    else if (p_dtype == MUON_HIP_BF16 && u_dtype == MUON_HIP_BF16)
+        hipLaunchKernelGGL((decay_update_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (bf16_t*)p, (const bf16_t*)u, n, decay, alpha);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();

@@ -15,6 +15,7 @@
 // Operands and results live in the blocked layout of common.h (256 x 32 blocks), zero padded
 // by the producers to whole tiles, so there is no masking here; the host launcher checks that
 // the shapes it is given are whole tiles before launching.
+#include <atomic>
 #include <type_traits>
 
 #include "common.h"
@@ -716,14 +717,14 @@ hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
     constexpr int stages = 2 * (BM + BN) * ROW_BYTES;
     constexpr int epi = EPI == EPI_BX ? epilogue_nn_bytes<BM, BN>() : epilogue_bytes<BM, BN>();
     constexpr int smem = stages > epi ? stages : epi;
-    static bool configured = false;  // per instantiation; the attribute is idempotent
+    static std::atomic<bool> configured{false};  // per instantiation; setting the attribute twice is harmless
     void (*kern)(const GemmArgs);
     if constexpr (FEED == 1) kern = gemm_nt_pp_kernel<BM, BN, WGM, WGN, EPI>;
     else kern = gemm_nt_pipe_kernel<BM, BN, WGM, WGN, EPI>;
-    if (!configured) {
+    if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
-        configured = true;
+        configured.store(true, std::memory_order_release);
     }
     hipLaunchKernelGGL(kern, dim3(nblocks), dim3(WGM * WGN * 64), smem, stream, g);
     return hipGetLastError();
@@ -755,12 +756,12 @@ hipError_t launch_pp_tail(GemmArgs g, int nblocks, int rest, hipStream_t stream)
     constexpr int stages = 2 * (256 + 256) * ROW_BYTES;
     constexpr int epi = EPI == EPI_BX ? epilogue_nn_bytes<256, 256>() : epilogue_bytes<256, 256>();
     constexpr int smem = stages > epi ? stages : epi;  // the 128-tiles need less of both
-    static bool configured = false;
+    static std::atomic<bool> configured{false};
     auto kern = gemm_nt_pp_tail_kernel<EPI>;
-    if (!configured) {
+    if (!configured.load(std::memory_order_acquire)) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
-        configured = true;
+        configured.store(true, std::memory_order_release);
     }
     g.big_blocks = nblocks - rest;
     hipLaunchKernelGGL(kern, dim3(g.big_blocks + 4 * rest), dim3(512), smem, stream, g);

@@ -88,14 +88,15 @@ struct AdamConst {
 };
 
 template <typename T>
-__device__ __forceinline__ void adam_one(float& p, float g, float& e1, float& e2, const AdamConst& am, float c1, float c2) {
+__device__ __forceinline__ void adam_one(float& p, float g, float& e1, float& e2, const AdamConst& am, float r1, float r2) {
     const float a = Mt<T>::rnd(lerp_aten(e1, g, am.w1, am.w1m1, am.small1));
     const float g2 = Mt<T>::rnd(g * g);
     const float bb = Mt<T>::rnd(lerp_aten(e2, g2, am.w2, am.w2m1, am.small2));
     e1 = a;
     e2 = bb;
-    const float ac = Mt<T>::rnd(__fdiv_rn(a, c1));
-    const float bc = Mt<T>::rnd(__fdiv_rn(bb, c2));
+    // a tensor divided by a python scalar is a multiplication by the scalar's fp32 reciprocal on a GPU
+    const float ac = Mt<T>::rnd(a * r1);
+    const float bc = Mt<T>::rnd(bb * r2);
     const float den = Mt<T>::rnd(Mt<T>::rnd(__fsqrt_rn(bc)) + am.eps);
     const float upd = Mt<T>::rnd(__fdiv_rn(ac, den));
     const float pd = Mt<T>::rnd(p * am.decay);
@@ -112,7 +113,7 @@ adamw_multi_kernel(const void* const* p_ptrs, const void* const* g_ptrs, const v
     const T* g = (const T*)g_ptrs[r.t] + r.begin;
     T* e1 = (T*)e1_ptrs[r.t] + r.begin;
     T* e2 = (T*)e2_ptrs[r.t] + r.begin;
-    const float c1 = (float)bias1[r.t], c2 = (float)bias2[r.t];
+    const float r1 = __fdiv_rn(1.0f, (float)bias1[r.t]), r2 = __fdiv_rn(1.0f, (float)bias2[r.t]);
     const bool vec = ((((uintptr_t)p) | ((uintptr_t)g) | ((uintptr_t)e1) | ((uintptr_t)e2)) & 15) == 0;
     const long n8 = vec ? r.len / 8 : 0;
     for (long i = threadIdx.x; i < n8; i += 256) {
@@ -122,14 +123,14 @@ adamw_multi_kernel(const void* const* p_ptrs, const void* const* g_ptrs, const v
         Mt<T>::load8(e1 + i * 8, av);
         Mt<T>::load8(e2 + i * 8, bv);
 #pragma unroll
-        for (int k = 0; k < 8; ++k) adam_one<T>(pv[k], gv[k], av[k], bv[k], am, c1, c2);
+        for (int k = 0; k < 8; ++k) adam_one<T>(pv[k], gv[k], av[k], bv[k], am, r1, r2);
         Mt<T>::store8(e1 + i * 8, av);
         Mt<T>::store8(e2 + i * 8, bv);
         Mt<T>::store8(p + i * 8, pv);
     }
     for (long i = n8 * 8 + threadIdx.x; i < r.len; i += 256) {
         float pv = Mt<T>::load(p + i), av = Mt<T>::load(e1 + i), bv = Mt<T>::load(e2 + i);
-        adam_one<T>(pv, Mt<T>::load(g + i), av, bv, am, c1, c2);
+        adam_one<T>(pv, Mt<T>::load(g + i), av, bv, am, r1, r2);
         Mt<T>::store(e1 + i, av);
         Mt<T>::store(e2 + i, bv);
         Mt<T>::store(p + i, pv);

@@ -15,6 +15,7 @@ Differences from the reference, all deliberate:
     they say.  The reference's single-device call site passes them swapped positionally
     (muon_utils.py:316-323 into :186); `reference_bug_compat=True` reproduces that.
   * p.grad is not overwritten with the Nesterov blend unless `write_back_grad=True`.
+  * the Newton-Schulz workspace is kept between steps (`keep_workspace=False` or `release_workspace()` frees it).
   * `momentum_dtype=torch.float32` keeps an fp32 momentum buffer for bf16 parameters (the
     reference always uses the parameter's dtype, muon_utils.py:450).
 """
@@ -34,6 +35,25 @@ from . import _abi
 logger = logging.getLogger(__name__)
 
 NS_COEFFS = (3.4445, -4.7750, 2.0315)  # muon_utils.py:137
+
+# Cap of the Newton-Schulz workspace one grouped launch may use; buckets that need more are cut into chunks.
+DEFAULT_WORKSPACE_LIMIT = 24 << 30
+
+_noted_semantics = False
+
+
+def _note_keyword_semantics() -> None:
+    """Once per process: this optimizer is not arithmetic-identical to the reference's single-device call site."""
+    global _noted_semantics
+    if _noted_semantics:
+        return
+    _noted_semantics = True
+    logger.warning(
+        "Muon (MI355X build): ns_steps and nesterov are honoured as named. The reference's single-device call site "
+        "passes them swapped (one Newton-Schulz iteration, Nesterov always on); pass reference_bug_compat=True to "
+        "reproduce that trajectory."
+    )
+
 
 _MUON_KEYS = {"params", "lr", "momentum", "weight_decay", "use_muon", "rms_scale", "nesterov", "ns_steps"}
 _ADAM_KEYS = {"params", "lr", "betas", "eps", "weight_decay", "use_muon"}
@@ -98,6 +118,33 @@ def matmul_transpose_assign(d_in: Tensor, d_out: Tensor) -> None:
             d_out.copy_(out)
 
 
+def get_autotune_config():
+    """muon_utils.py:13-25 lists the Triton tile shapes the autotuner tries.  The HIP kernels are not autotuned:
+    this returns the fixed tile configurations the launcher chooses between by shape."""
+    return [
+        dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, num_stages=2, num_warps=4, config=_abi.CFG_128_PIPE),
+        dict(BLOCK_SIZE_M=256, BLOCK_SIZE_N=256, BLOCK_SIZE_K=64, num_stages=2, num_warps=8, config=_abi.CFG_256_PIPE),
+        dict(BLOCK_SIZE_M=256, BLOCK_SIZE_N=256, BLOCK_SIZE_K=32, num_stages=4, num_warps=8, config=_abi.CFG_256_PINGPONG),
+    ]
+
+
+class _MmtKernel:
+    """Stands where the reference keeps its Triton kernel object (muon_utils.py:28-92) so that code which
+    launches it as `mmt_kernel[grid](x, y, M, K, stride_xm, stride_xk, stride_ym, stride_yn)` keeps working:
+    the launch runs the symmetric MFMA kernel through matmul_transpose_assign; the grid is ignored."""
+
+    def __getitem__(self, grid):
+        def launch(x, y, M, K, stride_xm, stride_xk, stride_ym, stride_yn, **meta):
+            src = torch.as_strided(x, (M, K), (stride_xm, stride_xk))
+            dst = torch.as_strided(y, (M, M), (stride_ym, stride_yn))
+            matmul_transpose_assign(src, dst)
+
+        return launch
+
+
+mmt_kernel = _MmtKernel()
+
+
 def matmul_transpose(d_in: Tensor) -> Tensor:
     M, _ = d_in.shape
     d_out = torch.empty((M, M), device=d_in.device, dtype=d_in.dtype)
@@ -153,9 +200,38 @@ def apply_momentum(grad: Tensor, momentum: Tensor, beta: float, nesterov: bool) 
 
 
 def apply_scaling(grad: Tensor, rms_scale: bool = False) -> Tensor:
-    """muon_utils.py:167-175.  A host-level helper; step() fuses this into the update kernel."""
-    grad *= scale_factor(grad.size(-2), grad.size(-1), rms_scale)
+    """muon_utils.py:167-175, in place, one rounding in grad's dtype.  step() fuses this into the update kernel;
+    this is the stand-alone helper."""
+    _require_cuda(grad, "grad")
+    if not grad.is_contiguous():
+        raise NotImplementedError("apply_scaling needs a contiguous tensor")
+    with torch.cuda.device(grad.device):
+        _abi.check(
+            _abi.lib().muon_hip_scale(grad.data_ptr(), _abi.dtype_code(grad.dtype), grad.numel(),
+                                      float(scale_factor(grad.size(-2), grad.size(-1), rms_scale)),
+                                      _abi.stream_ptr(grad.device)),
+            "scale",
+        )
     return grad
+
+
+def adam_update(grad: Tensor, buf1: Tensor, buf2: Tensor, step: int, betas, eps: float) -> Tensor:
+    """muon_utils.py:178-183: both moment buffers move in place, the bias-corrected update is returned."""
+    _require_cuda(grad, "grad")
+    if not (grad.dtype == buf1.dtype == buf2.dtype):
+        raise TypeError("adam_update: grad and both moment buffers must share one dtype")
+    if not (buf1.is_contiguous() and buf2.is_contiguous()) or grad.shape != buf1.shape or grad.shape != buf2.shape:
+        raise NotImplementedError("adam_update needs contiguous moment buffers of the gradient's shape")
+    g = grad if grad.is_contiguous() else grad.contiguous()
+    out = torch.empty_like(buf1)
+    with torch.cuda.device(grad.device):
+        _abi.check(
+            _abi.lib().muon_hip_adam_update(g.data_ptr(), buf1.data_ptr(), buf2.data_ptr(), out.data_ptr(),
+                                            _abi.dtype_code(grad.dtype), grad.numel(), int(step), float(betas[0]),
+                                            float(betas[1]), float(eps), _abi.stream_ptr(grad.device)),
+            "adam_update",
+        )
+    return out
 
 
 def muon_update(grad, momentum, beta=0.95, ns_steps=5, nesterov=True, rms_scale=False):
@@ -276,14 +352,18 @@ class Muon(torch.optim.Optimizer):
         momentum_dtype: Optional[torch.dtype] = None,
         reference_bug_compat: bool = False,
         write_back_grad: bool = False,
-        workspace_limit_bytes: int = 24 << 30,
+        workspace_limit_bytes: int = DEFAULT_WORKSPACE_LIMIT,
+        keep_workspace: bool = True,
     ):
         self.is_deepspeed_enabled = is_deepspeed_enabled
         self.momentum_dtype = momentum_dtype
         self.reference_bug_compat = reference_bug_compat
         self.write_back_grad = write_back_grad
         self.workspace_limit_bytes = int(workspace_limit_bytes)
+        self.keep_workspace = bool(keep_workspace)
         self._workspaces = {}
+        if not reference_bug_compat and not is_deepspeed_enabled:
+            _note_keyword_semantics()
         for group in param_groups:
             assert "use_muon" in group
             if group["use_muon"]:
@@ -334,10 +414,51 @@ class Muon(torch.optim.Optimizer):
 
     @torch.no_grad()
     def step_deepspeed(self, closure=None):
-        raise NotImplementedError(
-            "the DeepSpeed branch (muon_utils.py:395-432) relies on DeepSpeed's own ZeRO Muon and is not part of "
-            "this single-GPU build"
-        )
+        """muon_utils.py:395-432.  Under DeepSpeed the orthogonalised update already sits in p.grad, so a Muon group
+        only decays and updates (:405-407); the Adam groups run the same arithmetic as step_fsdp (the reference
+        imports DeepSpeed's copy of adam_update there, the formula of :178-183)."""
+        loss = None
+        if closure is not None:
+            with torch.enable_grad():
+                loss = closure()
+        lib = _abi.lib()
+        for group in self.param_groups:
+            if group["use_muon"]:
+                for p in group["params"]:
+                    _require_cuda(p, "a Muon parameter")
+                    if not p.is_contiguous():
+                        raise NotImplementedError("Muon parameters must be contiguous")
+                    u = p.grad.reshape(p.shape)
+                    u = u if u.is_contiguous() else u.contiguous()
+                    with torch.cuda.device(p.device):
+                        _abi.check(
+                            lib.muon_hip_decay_update(p.data_ptr(), _abi.dtype_code(p.dtype), u.data_ptr(),
+                                                      _abi.dtype_code(u.dtype), p.numel(), float(group["lr"]),
+                                                      float(group["weight_decay"]), _abi.stream_ptr(p.device)),
+                            "decay_update",
+                        )
+            else:
+                self._adam_group_step(group)
+        return loss
+
+    def release_workspace(self) -> None:
+        """Drop the Newton-Schulz workspace (it is re-allocated by the next step): for callers that want the
+        memory back between optimizer steps, e.g. for activations."""
+        self._workspaces.clear()
+
+    def _adam_group_step(self, group) -> None:
+        items = []
+        for p in group["params"]:
+            if p.grad is None:
+                p.grad = torch.zeros_like(p)
+            state = self.state[p]
+            if len(state) == 0:
+                state["exp_avg"] = torch.zeros_like(p)
+                state["exp_avg_sq"] = torch.zeros_like(p)
+                state["step"] = 0
+            state["step"] += 1
+            items.append((p, p.grad, state["exp_avg"], state["exp_avg_sq"], state["step"]))
+        _adamw_group(items, group)
 
     def load_state_dict(self, state_dict) -> None:
         """torch casts every floating state tensor to the parameter's dtype on load; put an
@@ -396,19 +517,10 @@ class Muon(torch.optim.Optimizer):
                     _muon_bucket_step(ps, gs, ms, group, ns_steps, nesterov, self.write_back_grad, self._workspaces,
                                       self.workspace_limit_bytes)
             else:
-                items = []
-                for p in group["params"]:
-                    if p.grad is None:
-                        p.grad = torch.zeros_like(p)
-                    state = self.state[p]
-                    if len(state) == 0:
-                        state["exp_avg"] = torch.zeros_like(p)
-                        state["exp_avg_sq"] = torch.zeros_like(p)
-                        state["step"] = 0
-                    state["step"] += 1
-                    items.append((p, p.grad, state["exp_avg"], state["exp_avg_sq"], state["step"]))
-                _adamw_group(items, group)
+                self._adam_group_step(group)
 
+        if not self.keep_workspace:
+            self.release_workspace()
         for work in dq:
             work.finish()
 

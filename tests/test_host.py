@@ -80,8 +80,61 @@ def test_deepspeed_quirks_kept():
     opt = Muon([g], is_deepspeed_enabled=True)
     assert g["rms_scale"] is False, "DeepSpeed forces rms_scale off"
     assert g["nesterov"] is False, "the reference warns but keeps False"
-    with pytest.raises(NotImplementedError):
-        opt.step()
+    g["params"][0].grad = torch.zeros(4, 3)
+    with pytest.raises(_abi.MuonHipError, match="no CPU path"):
+        opt.step()  # dispatches to step_deepspeed, which has no CPU path either
+
+
+# every top-level name of the reference module (muon_utils.py:13, 33, 95, 122, 129, 159, 167, 178, 186, 195, 206,
+# 278, 287, 296, 305, 331)
+REFERENCE_MODULE_NAMES = [
+    "get_autotune_config", "mmt_kernel", "matmul_transpose_assign", "matmul_transpose", "fast_newtonschulz",
+    "apply_momentum", "apply_scaling", "adam_update", "muon_update", "Work", "Fsdp1dWork", "TpFsdp2dWork",
+    "EpFsdp2dWork", "TpEpFsdp3dWork", "SingelDeviceWork", "Muon",
+]
+
+
+def test_module_substitution_is_name_complete(monkeypatch):
+    """Installing this module under the reference's import path: `from lmms_engine.utils.muon_utils import Muon`
+    (train/hf/trainer.py:459) then resolves here, and so does every other public name of the reference module."""
+    import importlib
+    import sys
+    import types
+
+    pkg, sub = types.ModuleType("lmms_engine"), types.ModuleType("lmms_engine.utils")
+    pkg.utils, sub.muon_utils = sub, muon_utils
+    monkeypatch.setitem(sys.modules, "lmms_engine", pkg)
+    monkeypatch.setitem(sys.modules, "lmms_engine.utils", sub)
+    monkeypatch.setitem(sys.modules, "lmms_engine.utils.muon_utils", muon_utils)
+    mod = importlib.import_module("lmms_engine.utils.muon_utils")
+    assert mod is muon_utils
+    from lmms_engine.utils.muon_utils import Muon as Swapped  # the factory's own import line
+
+    assert Swapped is Muon
+    for name in REFERENCE_MODULE_NAMES:
+        assert hasattr(mod, name), f"{name} is a public name of the reference module"
+    import inspect
+
+    assert list(inspect.signature(mod.adam_update).parameters) == ["grad", "buf1", "buf2", "step", "betas", "eps"]
+    assert list(inspect.signature(mod.muon_update).parameters) == ["grad", "momentum", "beta", "ns_steps", "nesterov", "rms_scale"]
+    assert list(inspect.signature(mod.apply_momentum).parameters) == ["grad", "momentum", "beta", "nesterov"]
+    assert list(inspect.signature(mod.Muon.__init__).parameters)[:4] == ["self", "param_groups", "defaults", "is_deepspeed_enabled"]
+    assert len(mod.get_autotune_config()) == 3
+
+
+def test_keyword_semantics_are_announced_once(caplog):
+    import logging
+
+    muon_utils._noted_semantics = False
+    with caplog.at_level(logging.WARNING, logger=muon_utils.logger.name):
+        Muon([dict(params=[P(4, 3)], use_muon=True)])
+        Muon([dict(params=[P(4, 3)], use_muon=True)])
+    assert sum("reference_bug_compat" in r.message for r in caplog.records) == 1
+    caplog.clear()
+    muon_utils._noted_semantics = False
+    with caplog.at_level(logging.WARNING, logger=muon_utils.logger.name):
+        Muon([dict(params=[P(4, 3)], use_muon=True)], reference_bug_compat=True)
+    assert not caplog.records
 
 
 def test_work_class_dispatch():
@@ -235,6 +288,12 @@ def test_argument_errors_are_reported_before_any_launch():
     rejected(lib.muon_hip_adamw(None, tbl, tbl, tbl, F32, 4, 1, 1e-3, 0.9, 0.95, 1e-8, 0.0, None), EINVAL, "null tensor")
     rejected(lib.muon_hip_adamw(tbl, tbl, tbl, tbl, F32, 4, 0, 1e-3, 0.9, 0.95, 1e-8, 0.0, None), EINVAL, "step")
     assert lib.muon_hip_adamw(tbl, tbl, tbl, tbl, F32, 0, 1, 1e-3, 0.9, 0.95, 1e-8, 0.0, None) == 0  # empty tensor
+    rejected(lib.muon_hip_adam_update(tbl, tbl, None, tbl, F32, 4, 1, 0.9, 0.95, 1e-8, None), EINVAL, "null tensor")
+    rejected(lib.muon_hip_adam_update(tbl, tbl, tbl, tbl, F32, 4, 0, 0.9, 0.95, 1e-8, None), EINVAL, "step")
+    rejected(lib.muon_hip_scale(None, F32, 4, 2.0, None), EINVAL, "null tensor")
+    rejected(lib.muon_hip_scale(tbl, 5, 4, 2.0, None), EINVAL, "dtype")
+    rejected(lib.muon_hip_decay_update(tbl, BF16, tbl, F32, 4, 0.02, 0.0, None), EINVAL, "fp32 update")
+    rejected(lib.muon_hip_decay_update(None, F32, tbl, F32, 4, 0.02, 0.0, None), EINVAL, "null tensor")
     rejected(lib.muon_hip_adamw_multi(tbl, tbl, tbl, tbl, tbl, tbl, tbl, tbl, 0, 1, F32, 1e-3, 0.9, 0.95, 1e-8, 0.0,
                                       None), EINVAL, "at least one tensor")
     rejected(lib.muon_hip_adamw_multi(tbl, tbl, tbl, tbl, tbl, tbl, None, tbl, 1, 1, F32, 1e-3, 0.9, 0.95, 1e-8, 0.0,
