@@ -26,11 +26,37 @@ if ROOT not in sys.path:
 METRIC = "Muon step ms + NS TFLOP/s (% bf16 MFMA peak), Qwen3-8B param set, 1 GPU"
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
-# Mean HBM-side bytes (L2 misses plus write-backs) of one B.X launch in a full step of each workload:
-# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE over this script, each scaled by what the same counter
-# reads for the 1 GiB copy of --calibrate-copy (one FETCH_SIZE unit = 2 KiB, one WRITE_SIZE unit = 1 KiB).
-# A counter run cannot share a process with the event timing, so the figure is carried here.
-BX_TRAFFIC_BYTES_PER_LAUNCH = {"qwen3-8b": 23.455e9 + 3.473e9}
+# Mean HBM-side bytes (L2 misses plus write-backs) of one B.X launch in a full step: rocprofv3 --pmc FETCH_SIZE
+# and --pmc WRITE_SIZE over this script, each scaled by what the same counter reads for the 1 GiB copy of
+# --calibrate-copy.  A counter run cannot share a process with the event timing, so the figure lives in the
+# tracked summary of that run, on a line
+#   roofline.traffic workload=<name> bytes_per_launch=<float> gemm_nt_hip_blob=<git blob hash of gemm_nt.hip>
+# and is reported only while the GEMM source is still the one it was measured on.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "muon_step_qwen3_8b_hbm_traffic.txt")
+GEMM_SOURCE = os.path.join(ROOT, "lmms_engine_amd", "csrc", "gemm_nt.hip")
+
+
+def git_blob_hash(path):
+    """What `git hash-object` prints for the file."""
+    import hashlib
+
+    data = open(path, "rb").read()
+    return hashlib.sha1(b"blob %d\0" % len(data) + data).hexdigest()
+
+
+def recorded_traffic(workload):
+    """bytes per B.X launch from the tracked counter summary, or None when absent or measured on other code."""
+    try:
+        cur = git_blob_hash(GEMM_SOURCE)
+        for line in open(TRAFFIC_SUMMARY):
+            if not line.lstrip("# ").startswith("roofline.traffic "):
+                continue
+            kv = dict(tok.split("=", 1) for tok in line.split()[1:] if "=" in tok)
+            if kv.get("workload") == workload and kv.get("gemm_nt_hip_blob") == cur:
+                return float(kv["bytes_per_launch"])
+    except (OSError, ValueError, KeyError):
+        pass
+    return None
 
 WORKLOADS = {
     "qwen3-8b": dict(layers=36, shapes=dict(q=(4096, 4096), k=(1024, 4096), v=(1024, 4096), o=(4096, 4096),
@@ -71,7 +97,16 @@ def cpu_baseline(w, layers, target_flops_per_step):
 
     from oracle import muon_oracle as O
 
+    # the GPU box gives one job 16 host cores, whatever os.cpu_count() shows there: the cap is the whole share
     torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
+    cpu_model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                cpu_model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
     counts = {}
     for s in matrix_list(w, layers):
         counts[s] = counts.get(s, 0) + 1
@@ -99,6 +134,8 @@ def cpu_baseline(w, layers, target_flops_per_step):
         "value": target_flops_per_step / total_s / 1e12,
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
+        "cpu_model": cpu_model,
+        "host_cores_visible": os.cpu_count(),
         "kind": "port",
         "step_s_extrapolated": total_s,
         "sample": "one full Muon step of the torch CPU oracle per (rows, cols) bucket "
@@ -144,6 +181,121 @@ def extras(params, pd, dev, reps):
     return res
 
 
+def _event_ms(fn, reps, torch):
+    """Mean milliseconds of fn() over `reps` calls after one warm-up call, from events on the current stream."""
+    fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def gpu_oracle(params, moms, shapes, flops_step, reps=2):
+    """The second baseline: the reference's own torch expressions (muon_utils.py:138-156, :188-189, :324-325) run
+    unfused on the same GPU, one parameter at a time, with torch's bf16 matmul (hipBLASLt) for every product,
+    X @ X.mT standing in for the Triton kernel.  Also the library GEMM alone on the shapes of the dominant kernel:
+    B (M x M) @ X (M x K) in bf16, as dense TFLOP/s, to set beside the B.X kernel's figure."""
+    import torch
+
+    a, b, c = 3.4445, -4.7750, 2.0315
+    beta, lr, wd, steps = HP["momentum"], HP["lr"], HP["weight_decay"], HP["ns_steps"]
+
+    def one(p, m):
+        g = p.grad if p.grad.dtype == m.dtype else p.grad.to(m.dtype)
+        m.lerp_(g, 1 - beta)
+        u = g.lerp(m, beta)
+        X = u.bfloat16()
+        if p.shape[0] > p.shape[1]:
+            X = X.mT
+        X = X / (X.norm(dim=(-2, -1), keepdim=True) + 1e-7)
+        for _ in range(steps):
+            A = X @ X.mT
+            A2 = A @ A.mT
+            B = b * A + c * A2
+            X = a * X + B @ X
+        if p.shape[0] > p.shape[1]:
+            X = X.mT
+        X = X * max(1, p.shape[0] / p.shape[1]) ** 0.5
+        p.mul_(1 - lr * wd)
+        p.add_(X.reshape(p.shape), alpha=-lr)
+
+    def step():
+        with torch.no_grad():
+            for p, m in zip(params, moms):
+                one(p, m)
+
+    ms = _event_ms(step, reps, torch)
+    dense = sum(HP["ns_steps"] * (4.0 * min(s) ** 2 * max(s) + 2.0 * min(s) ** 3) for s in shapes)
+    out = {"what": "reference expressions unfused in torch on this GPU (hipBLASLt bf16 matmuls, dense products)",
+           "ms_per_step": ms, "ns_tflops_algorithmic": flops_step / (ms * 1e-3) / 1e12,
+           "ns_tflops_dense_executed": dense / (ms * 1e-3) / 1e12}
+    dev = params[0].device
+    lib_gemm = {}
+    tot_f, tot_t = 0.0, 0.0
+    counts = {}
+    for s in shapes:
+        mk = (min(s), max(s))
+        counts[mk] = counts.get(mk, 0) + 1
+    for (M, K), cnt in sorted(counts.items()):
+        nb = max(1, min(cnt, 8, (2 << 30) // (M * K * 2)))
+        Bm = torch.randn(nb, M, M, device=dev).bfloat16() * 0.05
+        Xm = torch.randn(nb, M, K, device=dev).bfloat16() * 0.01
+        t_bx = _event_ms(lambda: [torch.matmul(Bm[i], Xm[i]) for i in range(nb)], 5, torch)
+        t_xx = _event_ms(lambda: [torch.matmul(Xm[i], Xm[i].mT) for i in range(nb)], 5, torch)
+        f = 2.0 * M * M * K * nb
+        lib_gemm[f"{M}x{K}"] = {"matrices": nb, "B@X_tflops": f / (t_bx * 1e-3) / 1e12,
+                                "X@X.mT_tflops_dense": f / (t_xx * 1e-3) / 1e12}
+        tot_f += 2.0 * M * M * K * cnt
+        tot_t += t_bx * 1e-3 / nb * cnt
+        del Bm, Xm
+    out["library_gemm"] = lib_gemm
+    out["library_B@X_tflops_weighted"] = tot_f / tot_t / 1e12
+    return out
+
+
+def operand_power(dev, M=4096, K=12288, nb=16, reps=10):
+    """The three product entry points on operands of one size, filled (a) with independent random values of the
+    magnitude the iteration sees and (b) with one constant: same kernels, same bytes, same instruction stream.
+    The difference is what the operand data costs (the part lowers its clock under matrix-pipe load)."""
+    import torch
+
+    from lmms_engine_amd import _abi
+
+    lib = _abi.lib()
+    nx, na = lib.muon_hip_blocked_elems(M, K), lib.muon_hip_blocked_elems(M, M)
+    X = torch.empty(nb * nx, dtype=torch.bfloat16, device=dev)
+    Xo = torch.empty_like(X)
+    A = torch.empty(nb * na, dtype=torch.bfloat16, device=dev)
+    Bm = torch.empty_like(A)
+    res = {}
+    for label in ("random", "constant"):
+        if label == "random":
+            X.copy_((torch.randn(nb * nx, device=dev) * (1.0 / K ** 0.5)).bfloat16())
+            A.copy_((torch.randn(nb * na, device=dev) * (1.0 / M ** 0.5)).bfloat16())
+        else:
+            X.fill_(1.0 / 128)
+            A.fill_(1.0 / 64)
+        calls = {
+            "syrk": (lambda: _abi.check(lib.muon_hip_syrk_bf16(X.data_ptr(), Bm.data_ptr(), M, K, nb, -1, _abi.stream_ptr(dev))),
+                     float(M) * M * K * nb),
+            "sympoly": (lambda: _abi.check(lib.muon_hip_sympoly_bf16(A.data_ptr(), Bm.data_ptr(), M, nb, -4.775, 2.0315, -1,
+                                                                     _abi.stream_ptr(dev))), float(M) ** 3 * nb),
+            "bx_axpy": (lambda: _abi.check(lib.muon_hip_bx_axpy_bf16(A.data_ptr(), X.data_ptr(), Xo.data_ptr(), M, K, nb, 3.4445,
+                                                                     -1, _abi.stream_ptr(dev))), 2.0 * M * M * K * nb),
+        }
+        res[label] = {}
+        for name, (fn, flop) in calls.items():
+            ms = _event_ms(fn, reps, torch)
+            res[label][name] = {"ms": ms, "tflops": flop / (ms * 1e-3) / 1e12,
+                                "frac_mfma_peak": flop / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+    res["shape"] = f"{nb} matrices {M}x{K}"
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -159,6 +311,15 @@ def main():
     ap.add_argument("--extras", action="store_true",
                     help="also time the two neighbours of the Muon step, outside the timed region: gradient-norm clipping "
                          "over the same gradients and the AdamW fallback over an embedding + lm_head + norm-vector group")
+    ap.add_argument("--no-gpu-oracle", action="store_true",
+                    help="skip the second baseline (the reference's expressions unfused in torch on this GPU, and the "
+                         "library bf16 GEMM on the shapes of the dominant kernel), which runs after the timed region")
+    ap.add_argument("--operand-power", action="store_true",
+                    help="also time the three product entry points on random and on constant operands of one size")
+    ap.add_argument("--operand-power-only", action="store_true",
+                    help="run only the --operand-power measurement (for counter runs)")
+    ap.add_argument("--gemm-config", type=int, default=-1,
+                    help="force one GEMM tile configuration (MUON_HIP_CFG_*; -1 = chosen per kernel and shape)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device copy (a kernel of known traffic) so that FETCH_SIZE / WRITE_SIZE "
                          "readings of a rocprofv3 --pmc run can be scaled")
@@ -179,6 +340,11 @@ def main():
         build_library()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    if args.gemm_config >= 0:
+        _abi.check(_abi.lib().muon_hip_set_gemm_config(args.gemm_config), "set_gemm_config")
+    if args.operand_power_only:
+        print(json.dumps({"operand_power": operand_power(dev)}))
+        return
     w = WORKLOADS[args.workload]
     layers = args.layers or w["layers"]
     shapes = matrix_list(w, layers)
@@ -208,12 +374,18 @@ def main():
     torch.cuda.synchronize()
     if not args.no_kernel_timing:
         _abi.timing_enable(True)
+    # one event per step boundary on the stream the kernels run on: per-step times for the median and the minimum
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    marks[0].record()
+    for i in range(args.steps):
         opt.step()
+        marks[i + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_step = dt / args.steps * 1e3
+    step_ms = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    ms_median = step_ms[len(step_ms) // 2] if len(step_ms) % 2 else 0.5 * (step_ms[len(step_ms) // 2 - 1] + step_ms[len(step_ms) // 2])
     kern = {}
     if not args.no_kernel_timing:
         kern = _abi.timing_read()
@@ -248,7 +420,7 @@ def main():
         achieved = bx_f * args.steps / (tot_ms * 1e-3) / 1e12
         roofline = {"kernel": "gemm_nt_pp_kernel<256, 256, 2, 4, EPI_BX> (X' = a.X + B.X)", "bound": "mfma", "achieved": achieved,
                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                    "traffic": BX_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload) if layers == w["layers"] else None,
+                    "traffic": recorded_traffic(args.workload) if layers == w["layers"] else None,
                     "launches": cnt, "avg_launch_ms": tot_ms / cnt,
                     "algorithmic_flop_per_launch": bx_f * args.steps / cnt}
     gemm_ms = sum(kernels[k]["ms_per_step"] for k in ("syrk", "sympoly", "bx_axpy") if k in kernels)
@@ -261,6 +433,9 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_step,
+        "ms_per_step_median": ms_median,
+        "ms_per_step_min": step_ms[0],
+        "ms_per_step_max": step_ms[-1],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -277,6 +452,13 @@ def main():
     }
     if args.extras:
         out["extras"] = extras(params, pd, dev, args.steps)
+    if args.operand_power:
+        out["operand_power"] = operand_power(dev)
+    if not args.no_gpu_oracle:
+        moms = [opt.state[p]["momentum_buffer"] for p in params]
+        out["gpu_oracle"] = gpu_oracle(params, moms, shapes, flops_step)
+        if roofline is not None:
+            out["gpu_oracle"]["bx_axpy_kernel_tflops"] = roofline["achieved"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w, layers, flops_step)
     print(json.dumps(out))

@@ -56,7 +56,8 @@ extern "C" {
 #define MUON_HIP_CFG_128_PIPE 0      /* 128x128 tile, 4 waves, 64-column k-tiles, two LDS stages */
 #define MUON_HIP_CFG_256_PIPE 1      /* 256x256 tile, 8 waves, the same pipeline */
 #define MUON_HIP_CFG_256_PINGPONG 2  /* 256x256 tile, two groups of 4 waves alternating memory / MFMA phases */
-#define MUON_HIP_CFG_COUNT 3
+#define MUON_HIP_CFG_256_PIPE4W 3    /* 256x256 tile, 4 waves of 128x128 (one per SIMD), the two-stage pipeline */
+#define MUON_HIP_CFG_COUNT 4
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);
@@ -204,6 +205,17 @@ int muon_hip_adamw_multi(const void* const* p_ptrs, const void* const* g_ptrs, c
 int muon_hip_grad_norms(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
                         int dtype, float* partials, float* norms, void* stream);
 int muon_hip_total_norm(const float* norms, int n, int dtype, float* total_f32, void* total_typed, void* stream);
+
+/* muon_hip_grad_norms without the `partials` argument.  No counterpart in the reference: it is for callers
+ * that cannot allocate device memory for the scratch buffer (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  The partial sums go to an array of MUON_HIP_STATIC_MAX_CHUNKS
+ * floats (4 MiB) built into the library, one copy per device, held until the process ends; more chunks than
+ * that are rejected with MUON_HIP_ESHAPE.  The call allocates and frees nothing.  All calls on one device share
+ * the array, so calls that may overlap on one device (different streams, different threads) race: serialise
+ * them.  The first call on a device looks the array's address up and must not run under stream capture. */
+#define MUON_HIP_STATIC_MAX_CHUNKS (1 << 20)
+int muon_hip_grad_norms_static(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n,
+                               long chunks, int dtype, float* norms, void* stream);
 int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
                         int dtype, const float* total_f32, int norm_dtype, double max_norm, void* stream);
 

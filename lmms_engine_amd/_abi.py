@@ -15,12 +15,13 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmuon_hip.so")
 
 F32, BF16 = 0, 1
-CFG_AUTO, CFG_128_PIPE, CFG_256_PIPE, CFG_256_PINGPONG = -1, 0, 1, 2
-GEMM_CONFIGS = list(range(3))
+CFG_AUTO, CFG_128_PIPE, CFG_256_PIPE, CFG_256_PINGPONG, CFG_256_PIPE4W = -1, 0, 1, 2, 3
+GEMM_CONFIGS = list(range(4))
 K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW, K_ADAMW_MULTI, K_GRAD_NORM, K_CLIP_SCALE = range(10)
 KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw", "adamw_multi",
                 "grad_norm", "clip_scale"]
 MULTI_CHUNK = 16384  # MUON_HIP_MULTI_CHUNK
+STATIC_MAX_CHUNKS = 1 << 20  # MUON_HIP_STATIC_MAX_CHUNKS
 
 # name -> (restype, argtypes); mirrors include/muon_hip.h one to one
 SIGNATURES = {
@@ -54,6 +55,7 @@ SIGNATURES = {
     "muon_hip_decay_update": (c_int, [c_void_p, c_int, c_void_p, c_int, c_long, c_double, c_double, c_void_p]),
     "muon_hip_adamw_multi": (c_int, [c_void_p] * 8 + [c_int, c_long, c_int] + [c_double] * 5 + [c_void_p]),
     "muon_hip_grad_norms": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_void_p, c_void_p]),
+    "muon_hip_grad_norms_static": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_void_p]),
     "muon_hip_total_norm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "muon_hip_clip_scale": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_int, c_double,
                                     c_void_p]),

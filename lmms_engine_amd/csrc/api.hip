@@ -484,6 +484,52 @@ int muon_hip_grad_norms(const void* const* g_ptrs, const long* numel, const long
     return e == hipSuccess ? 0 : hip_fail(e, "grad_norms launch");
 }
 
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// Partial sums of muon_hip_grad_norms_static live in this array instead of a caller buffer.  Each device the
+// library runs on holds its own copy at its own address, looked up once per device.
+static __device__ __align__(256) float scratch[MUON_HIP_STATIC_MAX_CHUNKS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device (0 on failure, with the error recorded).
+int scratch_for_current_device(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+    if (dev < 0 || dev >= kMaxDevices) return fail(MUON_HIP_EINVAL, "device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        float* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+        if (!ptr) return fail(MUON_HIP_EINVAL, "hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+}  // namespace
+
+int muon_hip_grad_norms_static(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n,
+                               long chunks, int dtype, float* norms, void* stream) {
+    if (int rc = check_list(g_ptrs, numel, chunk_start, n, chunks, dtype)) return rc;
+    if (!norms) return fail(MUON_HIP_EINVAL, "null output");
+    if (chunks > (long)MUON_HIP_STATIC_MAX_CHUNKS)
+        return fail(MUON_HIP_ESHAPE, "%ld chunks exceed the %ld the built-in scratch array holds; use muon_hip_grad_norms "
+                    "with a caller buffer", chunks, (long)MUON_HIP_STATIC_MAX_CHUNKS);
+    float* partials = nullptr;
+    if (int rc = scratch_for_current_device(&partials)) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    Timed t(MUON_HIP_K_GRAD_NORM, s);
+    const MultiTensorList l{g_ptrs, numel, chunk_start, n, chunks};
+    // every partial the second kernel reads is written by the first: nothing has to start at zero
+    hipError_t e = launch_tensor_norms(l, dtype, partials, norms, s);
+    return e == hipSuccess ? 0 : hip_fail(e, "grad_norms launch");
+}
+
 int muon_hip_total_norm(const float* norms, int n, int dtype, float* total_f32, void* total_typed, void* stream) {
     if (!norms || !total_f32 || !total_typed || n <= 0 || !dtype_ok(dtype))
         return fail(MUON_HIP_EINVAL, "null pointer, empty list or unknown dtype");

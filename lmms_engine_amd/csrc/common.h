@@ -41,6 +41,17 @@ __device__ __forceinline__ float bf2f(bf16_t h) { return (float)h; }
 // round through bf16 and return the fp32 value
 __device__ __forceinline__ float rbf(float f) { return (float)((bf16_t)f); }
 
+// Square roots and divisions: sqrtf(x) and __fdiv_rn(x, y) are correctly rounded in this build (hipcc's default
+// -fhip-fp32-correctly-rounded-divide-sqrt), which is what torch's GPU kernels compute; __fsqrt_rn is the
+// hardware approximation despite its name (it differs from the exact root in one result out of six) and is not used.
+
+// A value that the reference holds in a tensor of its own: the compiler must round it where it stands and not
+// contract the product behind it into the next addition (hipcc fuses across statements by default).
+__device__ __forceinline__ float materialized(float x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);

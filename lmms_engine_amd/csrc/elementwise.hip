@@ -197,7 +197,7 @@ __global__ void __launch_bounds__(256) frob_finalize_kernel(const float* partial
     for (int i = threadIdx.x; i < nparts; i += 256) s += partials[(long)b * nparts + i];
     s = block_sum_256(s, red);
     if (threadIdx.x == 0) {
-        const float nrm = rbf(__fsqrt_rn(s));
+        const float nrm = rbf(sqrtf(s));
         denom[b] = rbf(nrm + 1e-7f);
     }
 }
@@ -439,13 +439,13 @@ struct AdamMath {
 template <typename T>
 __device__ __forceinline__ float adam_moments(float gi, float& e1, float& e2, const AdamMath& am) {
     const float a = Ld<T>::rnd(lerp_aten(e1, gi, am.w1, am.w1m1, am.small1));
-    const float g2 = Ld<T>::rnd(gi * gi);
+    const float g2 = materialized(Ld<T>::rnd(gi * gi));  // grad.square() is a tensor of its own
     const float bb = Ld<T>::rnd(lerp_aten(e2, g2, am.w2, am.w2m1, am.small2));
     e1 = a;
     e2 = bb;
     const float ac = Ld<T>::rnd(a * am.r1);
     const float bc = Ld<T>::rnd(bb * am.r2);
-    const float den = Ld<T>::rnd(Ld<T>::rnd(__fsqrt_rn(bc)) + am.eps);
+    const float den = Ld<T>::rnd(Ld<T>::rnd(sqrtf(bc)) + am.eps);
     return Ld<T>::rnd(__fdiv_rn(ac, den));
 }
 
@@ -546,6 +546,7 @@ hipError_t launch_momentum_norm(const void* const* g_ptrs, const void* const* m_
     lerp_consts(1.0 - beta, mm.w1, mm.w1m1, mm.small1);
     lerp_consts(beta, mm.w2, mm.w2m1, mm.small2);
     mm.nesterov = nesterov != 0;
+    if (!mm.nesterov) write_back = 0;  // without Nesterov the update is the momentum buffer and the gradient stays as it is
     dim3 grid(nparts, batch), block(256);
     if (g_dtype == MUON_HIP_F32 && m_dtype == MUON_HIP_F32)
         hipLaunchKernelGGL((momentum_norm_kernel<float, float>), grid, block, 0, stream, g_ptrs, m_ptrs, U, strideU,

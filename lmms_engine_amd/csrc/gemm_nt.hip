@@ -1,4 +1,11 @@
-// GEMM family for the Newton-Schulz chain on gfx950 (v_mfma_f32_32x32x16_bf16).
+// GEMM family for the Newton-Schulz chain on gfx950, built on v_mfma_f32_16x16x32_bf16.
+//
+// Why the 16x16x32 instruction: under matrix-pipe load the part lowers its clock to stay inside its power
+// limit, and on operands with random mantissas a loop of nothing but 32x32x16 MFMAs sustains about 1.3 PFLOP/s
+// while the same loop of 16x16x32 MFMAs sustains about 2.05 (both reach 2.4 on constant operands): the deeper
+// dot product updates each fp32 accumulator half as often per FLOP.  Operand fragment: lane l holds row l%16,
+// eight consecutive k from 8*(l/16) (16 bytes).  Accumulator fragment: lane l holds column l%16, rows
+// 4*(l/16)+0..3 (f32x4).
 //
 // The three products of one NS iteration:
 //   SYRK     A  = bf(X Xt)                         P = Q = X   (M x K)           C[i][j] = sum_k P[i][k] Q[j][k]
@@ -27,27 +34,21 @@ namespace {
 // ~32 tiles an XCD works on at a time touch few distinct row panels.
 template <int GM>
 __device__ __forceinline__ void tri_decode(int t, int T, int& ti, int& tj) {
-    int r0 = 0;
-    for (;;) {
-        const int gm = (T - r0 < GM) ? (T - r0) : GM;
-        const int cnt = gm * (T - r0) - gm * (gm - 1) / 2;
-        if (t < cnt || r0 + gm >= T) {
-            const int tri = gm * (gm + 1) / 2;
-            if (t < tri) {
-                int c = 0;  // column c of the leading gm x gm triangle holds c+1 tiles
-                while (t >= c + 1) { t -= c + 1; ++c; }
-                ti = r0 + t;
-                tj = r0 + c;
-            } else {
-                t -= tri;
-                tj = r0 + gm + t / gm;
-                ti = r0 + t % gm;
-            }
-            return;
-        }
+    int r0 = 0, gm, cnt;
+    for (;;) {  // find the row group that holds tile t
+        gm = (T - r0 < GM) ? (T - r0) : GM;
+        cnt = gm * (T - r0) - gm * (gm - 1) / 2;
+        if (t < cnt || r0 + gm >= T) break;
         t -= cnt;
         r0 += gm;
     }
+    const int tri = gm * (gm + 1) / 2;
+    int c = 0, u = t;  // column c of the leading gm x gm triangle holds c+1 tiles
+    while (u >= c + 1 && c < gm - 1) { u -= c + 1; ++c; }
+    const int rest = t - tri;
+    const bool in_tri = t < tri;
+    ti = r0 + (in_tri ? u : rest % gm);
+    tj = r0 + (in_tri ? c : gm + rest / gm);
 }
 
 template <int GM>
@@ -77,12 +78,12 @@ __device__ __forceinline__ const T* uniform_ptr(const T* p) {
 // Tile `logical` (0 .. tiles_per_mat * batch - 1) in the launch order: matrix by matrix, 4-row groups.
 template <int EPI>
 __device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int logical) {
-    TileCoord tc;
-    tc.bidx = logical / g.tiles_per_mat;
-    const int t = logical - tc.bidx * g.tiles_per_mat;
-    if (EPI == EPI_BX) rect_decode<4>(t, g.tiles_m, g.tiles_n, tc.ti, tc.tj);
-    else tri_decode<4>(t, g.tiles_m, tc.ti, tc.tj);
-    return tc;
+    const int bidx = logical / g.tiles_per_mat;
+    const int t = logical - bidx * g.tiles_per_mat;
+    int ti = 0, tj = 0;  // plain locals: references into the struct kept it in scratch memory
+    if (EPI == EPI_BX) rect_decode<4>(t, g.tiles_m, g.tiles_n, ti, tj);
+    else tri_decode<4>(t, g.tiles_m, ti, tj);
+    return TileCoord{bidx, ti, tj};
 }
 
 template <int EPI>
@@ -107,8 +108,8 @@ __device__ __forceinline__ long panel_offset(int row0, int cb) {
 // One LDS copy of the tile, both output orientations written as 16-byte vectors.  The tile
 // lives in LDS as Tt[n][m] (n = local column, m = local row of the accumulator tile), the
 // orientation of Ct and of the elementwise source Et.  Every lane writes its rounded accumulators
-// as 8-byte pieces (4 consecutive m of one n, exactly what an accumulator lane holds: lane&31 owns
-// column n, registers 4q..4q+3 are rows 8q + 4*(lane>>5) + 0..3); after one barrier rows of Tt
+// as 8-byte pieces (4 consecutive m of one n, exactly what an accumulator lane holds: lane&15 owns
+// column n, its four registers are rows 4*(lane>>4) + 0..3 of the 16x16 fragment); after one barrier rows of Tt
 // leave as rows of Ct (SYMPOLY adds the b.A term there, from pieces of Et that each thread loaded
 // into registers before the accumulators were written, and puts the sums back), while rows of C
 // are gathered with ds_read_b64_tr_b16: in a group of 16 lanes, lane i receives element i%4 of the
@@ -128,15 +129,15 @@ __device__ __forceinline__ s16x4 lds_read_tr16(const unsigned char* p) {
 
 template <int BM, int BN, int WGM, int WGN, int EPI, bool MASKED>
 __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
-                                         f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], unsigned char* smem) {
+                                         f32x4 (&acc)[BM / WGM / 16][BN / WGN / 16], unsigned char* smem) {
     constexpr int NT = WGM * WGN * 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
-    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int FM = WTM / 16, FN = WTN / 16;
     constexpr int S = BM * 2 + 16;      // Tt row pitch (bytes): conflict-free for the 8-byte pieces
     constexpr int NLE = BN * (BM / 8) / NT;  // 16-byte chunks per thread for a whole tile
     static_assert((BN * (BM / 8)) % NT == 0 && BM % 64 == 0, "even split");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN, hi = lane >> 5;
+    const int wm = wave / WGN, wn = wave % WGN, quad = lane >> 4;
     const int m0 = tc.ti * BM, n0 = tc.tj * BN;
     const bool diag = (EPI != EPI_BX) && (tc.ti == tc.tj);
     // Et and Ct hold the tile as rows n0.. (BN of them) x columns m0.. (BM of them).  Chunk c of a
@@ -170,18 +171,16 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j)
+        for (int j = 0; j < FN; ++j) {
+            bf16x4 o;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                bf16x4 o;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float v = rbf(acc[i][j][q * 4 + r]);
-                    if (EPI == EPI_SYMPOLY) v = g.s1 * v;
-                    o[r] = f2bf(v);
-                }
-                *(bf16x4*)(smem + (wn * WTN + j * 32 + (lane & 31)) * S + (wm * WTM + i * 32 + q * 8 + hi * 4) * 2) = o;
+            for (int r = 0; r < 4; ++r) {
+                float v = rbf(acc[i][j][r]);
+                if (EPI == EPI_SYMPOLY) v = g.s1 * v;
+                o[r] = f2bf(v);
             }
+            *(bf16x4*)(smem + (wn * WTN + j * 16 + (lane & 15)) * S + (wm * WTM + i * 16 + quad * 4) * 2) = o;
+        }
     __syncthreads();
     {
         // rows of Tt leave as rows of Ct; SYMPOLY adds the rounded b.A term here and, when the tile itself is
@@ -229,8 +228,8 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
 }
 
 // Epilogue of BX.  The accumulators were built with the MFMA operands swapped, so a lane holds 4
-// consecutive columns n of one row m (lane&31 owns row m of its P fragment, registers 4q..4q+3 are columns
-// 8q + 4*(lane>>5) + 0..3 of its Q fragment): 8-byte pieces of rows of X'.  Every thread first issues the
+// consecutive columns n of one row m (lane&15 owns row m of its P fragment, its four registers are columns
+// 4*(lane>>4) + 0..3 of its Q fragment): 8-byte pieces of rows of X'.  Every thread first issues the
 // loads of its share of the a.X tile (16-byte pieces of rows, the layout of the output pass) into registers,
 // then the rounded accumulators go to LDS as T[m][n] while those loads are in flight; after one barrier each
 // thread reads its pieces of T, adds the rounded a.X term and stores rows of X' (1 KB contiguous per wave
@@ -240,16 +239,16 @@ constexpr int epilogue_nn_bytes() { return BM * (BN * 2 + 16); }
 
 template <int BM, int BN, int WGM, int WGN>
 __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& tc,
-                                            f32x16 (&acc)[BM / WGM / 32][BN / WGN / 32], unsigned char* smem) {
+                                            f32x4 (&acc)[BM / WGM / 16][BN / WGN / 16], unsigned char* smem) {
     constexpr int NT = WGM * WGN * 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
-    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int FM = WTM / 16, FN = WTN / 16;
     constexpr int S = BN * 2 + 16;           // T row pitch (bytes)
     constexpr int CPB = BLK_COLS / 8;        // 16-byte chunks per row of a block
     constexpr int NLE = BM * (BN / 8) / NT;  // 16-byte chunks per thread for a whole tile
     static_assert((BM * (BN / 8)) % NT == 0 && BN % BLK_COLS == 0, "even split");
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WGN, wn = wave % WGN, hi = lane >> 5;
+    const int wm = wave / WGN, wn = wave % WGN, quad = lane >> 4;
     const int m0 = tc.ti * BM, n0 = tc.tj * BN;
     // chunk c: 16 bytes j of the row piece of row m in column block cbk of the tile; a wave covers 16 rows of
     // one block = 1 KB contiguous in memory
@@ -271,14 +270,12 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j)
+        for (int j = 0; j < FN; ++j) {
+            bf16x4 t;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                bf16x4 t;
-#pragma unroll
-                for (int r = 0; r < 4; ++r) t[r] = f2bf(acc[i][j][q * 4 + r]);
-                *(bf16x4*)(smem + (wm * WTM + i * 32 + (lane & 31)) * S + (wn * WTN + j * 32 + q * 8 + hi * 4) * 2) = t;
-            }
+            for (int r = 0; r < 4; ++r) t[r] = f2bf(acc[i][j][r]);
+            *(bf16x4*)(smem + (wm * WTM + i * 16 + (lane & 15)) * S + (wn * WTN + j * 16 + quad * 4) * 2) = t;
+        }
     __syncthreads();
     bf16_t* C = g.C + tc.bidx * g.strideC;
 #pragma unroll
@@ -295,14 +292,17 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
 }
 
 // Transposing LDS read of a Q fragment of BX: the stage holds the k-tile of X as pieces of 32 columns,
-// [piece][k][32 columns] with 64-byte rows.  In a group of 16 lanes, lane j = 4r+s addresses row k+r, columns
-// 4s..4s+3 of the group's 16 columns and lane i = 4s+e receives rows k..k+3 of column 4s+e; the second read takes
-// rows k+4..k+7.  Lanes 16..31 take the upper 16 columns and lanes 32..63 rows k+8.., which is the MFMA operand
-// layout (lane l: row l%32 of the fragment, eight consecutive k from 8*(l/32)).  q points at row k of the piece
-// plus qt_lane_offset(lane).
-__device__ __forceinline__ int qt_lane_offset(int lane) {
+// [piece][k][32 columns] with 64-byte rows, and a fragment is 16 columns x 32 k.  ds_read_b64_tr_b16 works in
+// groups of 16 lanes: lane j = 4r+s addresses row k+r, columns 4s..4s+3 of the group's 16 columns, and lane
+// i = 4s+e receives rows k..k+3 of column 4s+e; a second read takes rows k+4..k+7.  Group g = lane/16 starts at
+// k = 8g, which gives the MFMA operand layout (lane l: column l%16, eight consecutive k from 8*(l/16)).
+// Two groups that are served together (g and g^1) would read the same 32-byte window of rows 64*8 bytes = two
+// bank rounds apart, so the two 32-byte halves of a row are stored swapped in rows whose k has bit 3 set (the
+// global side of the load applies the swap): fragment half h of group g sits at byte (h ^ (g & 1)) * 32.
+// qt_lane_offset(lane, h): byte offset of this lane's first read inside the piece, k-step 0.
+__device__ __forceinline__ int qt_lane_offset(int lane, int h) {
     const int grp = lane >> 4, i16 = lane & 15;
-    return ((grp >> 1) * 8 + (i16 >> 2)) * 64 + (grp & 1) * 32 + (i16 & 3) * 8;
+    return (grp * 8 + (i16 >> 2)) * 64 + ((h ^ (grp & 1)) * 32) + (i16 & 3) * 8;
 }
 __device__ __forceinline__ bf16x8 lds_read_qt(const unsigned char* q) {
     const s16x4 lo = lds_read_tr16(q), hi4 = lds_read_tr16(q + 4 * 64);
@@ -310,18 +310,22 @@ __device__ __forceinline__ bf16x8 lds_read_qt(const unsigned char* q) {
     return *(const bf16x8*)&t;
 }
 
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
 // ---- kernel 1: 64-column k-tiles in two LDS stages, one barrier per k-tile -------------------
 // Operand panels go from global memory straight into LDS (global_load_lds_dwordx4): one wave
 // instruction fills 1 KB of LDS in lane order, i.e. 8 rows of 128 bytes, so the XOR swizzle
 // that keeps the fragment reads conflict free (16-byte chunk c of row r sits at c ^ ((r>>1)&7))
 // is applied on the global side: lane L fetches the chunk whose swizzled position is L&7.
-// Per k-tile a wave issues FM*FN*4 MFMAs, (FM+FN)*4 LDS fragment reads and LA+LB loads.
-// Every non-MFMA instruction is placed between two MFMAs so that it issues in their shadow:
-//   k-steps 0..2 : MFMAs of step s interleaved with the fragment reads of step s+1;
-//   k-step 3     : the wave has now read everything it needs from this stage, so it waits
-//                  for its own loads of the next k-tile, crosses the one barrier, and then
-//                  interleaves the last MFMAs with the loads of k-tile t+2 (into the stage just
-//                  released) and with the fragment reads of step 0 of k-tile t+1.
+// Per k-tile (two 32-column MFMA steps) a wave issues FM*FN*2 MFMAs, (FM+FN)*2 LDS fragment reads and
+// LA+LB loads.  Every non-MFMA instruction is placed between two MFMAs so that it issues in their shadow:
+//   k-step 0 : MFMAs of step 0 interleaved with the fragment reads of step 1;
+//   k-step 1 : the wave has now read everything it needs from this stage, so it waits
+//              for its own loads of the next k-tile, crosses the one barrier, and then
+//              interleaves the last MFMAs with the loads of k-tile t+2 (into the stage just
+//              released) and with the fragment reads of step 0 of k-tile t+1.
 // The fences (sched_barrier) pin that order; without them the scheduler sinks every LDS read
 // next to its first use and the MFMA pipe idles for an LDS round trip per k-step.  Barriers are
 // raw s_barrier with explicit s_waitcnt: __syncthreads() would wait for the loads in flight.
@@ -331,10 +335,10 @@ template <int BM, int BN, int WGM, int WGN, int EPI>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmArgs g) {
     constexpr int NW = WGM * WGN;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
-    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int FM = WTM / 16, FN = WTN / 16;
     constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES, STAGE = A_BYTES + B_BYTES;
     constexpr int LA = BM / 8 / NW, LB = BN / 8 / NW;
-    constexpr int KS = 4;  // 16-column MFMA steps per k-tile
+    constexpr int KS = 2;  // 32-column MFMA steps per k-tile
     constexpr int NMF = FM * FN, NRD = FM + FN, NLD = LA + LB;
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "dma split");
     static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
@@ -354,8 +358,10 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     const int drow = lane >> 3;
     const bf16_t* pa = Pb + (wave * 8 * LA + drow) * BLK_COLS;
     // BX: a k-tile of Q is BN/32 pieces of 64 rows x 32 columns, each a contiguous 4 KB run of one block;
-    // load instruction t of the tile (1 KB) is the quarter t%4 of piece t/4, in lane order
-    const bf16_t* pb = QT ? Qb + (lane >> 2) * BLK_COLS + (lane & 3) * 8 : Qb + (wave * 8 * LB + drow) * BLK_COLS;
+    // load instruction t of the tile (1 KB) is the quarter t%4 of piece t/4, in lane order, with the two halves
+    // of a row swapped in rows whose k has bit 3 set (see qt_lane_offset)
+    const bf16_t* pb = QT ? Qb + (lane >> 2) * BLK_COLS + ((lane & 3) ^ (((lane >> 5) & 1) << 1)) * 8
+                          : Qb + (wave * 8 * LB + drow) * BLK_COLS;
     const int lds_a = wave * 8 * LA * ROW_BYTES;
     const int lds_b = A_BYTES + wave * 8 * LB * ROW_BYTES;
     // element offset of the 16-byte chunk this lane fetches inside a row of the 64-column k-tile, as an offset
@@ -383,32 +389,34 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
         }
     };
 
-    f32x16 acc[FM][FN];
+    f32x4 acc[FM][FN];
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    const int sw = (lane >> 1) & 7, hi = lane >> 5;
-    const int a_off = (wm * WTM + (lane & 31)) * ROW_BYTES;
-    const int b_off = QT ? A_BYTES + (wn * WTN / 32) * 4096 + qt_lane_offset(lane)
-                         : A_BYTES + (wn * WTN + (lane & 31)) * ROW_BYTES;
+    // fragment reads: lane l takes row l%16 of the fragment, 16-byte chunk 4*ks + l/16 of the 128-byte row
+    const int sw = (lane >> 1) & 7, kq = lane >> 4;
+    const int a_off = (wm * WTM + (lane & 15)) * ROW_BYTES;
+    const int b_off = A_BYTES + (wn * WTN + (lane & 15)) * ROW_BYTES;
+    const int q_off[2] = {A_BYTES + (wn * WTN / 32) * 4096 + qt_lane_offset(lane, 0),
+                          A_BYTES + (wn * WTN / 32) * 4096 + qt_lane_offset(lane, 1)};
 
     bf16x8 fr[2][NRD];  // fragment double buffer: [0..FM) rows of P, [FM..NRD) rows (BX: columns) of Q
     auto read_one = [&](int buf, int n, const unsigned char* st, int ks) {
-        const int co = (((ks << 1) | hi) ^ sw) << 4;
-        if (n < FM) fr[buf][n] = *(const bf16x8*)(st + a_off + n * 32 * ROW_BYTES + co);
-        else if (QT) fr[buf][n] = lds_read_qt(st + b_off + (n - FM) * 4096 + ks * 16 * 64);
-        else fr[buf][n] = *(const bf16x8*)(st + b_off + (n - FM) * 32 * ROW_BYTES + co);
+        const int co = (((ks << 2) | kq) ^ sw) << 4;
+        if (n < FM) fr[buf][n] = *(const bf16x8*)(st + a_off + n * 16 * ROW_BYTES + co);
+        else if (QT) fr[buf][n] = lds_read_qt(st + q_off[(n - FM) & 1] + ((n - FM) >> 1) * 4096 + ks * 32 * 64);
+        else fr[buf][n] = *(const bf16x8*)(st + b_off + (n - FM) * 16 * ROW_BYTES + co);
     };
     auto mfma_one = [&](int buf, int idx) {
         const int i = idx / FN, j = idx % FN;
         if (QT)  // operands swapped: a lane then holds 4 consecutive columns of one row of the tile
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[buf][FM + j], fr[buf][i], acc[i][j], 0, 0, 0);
+            acc[i][j] = mfma16(fr[buf][FM + j], fr[buf][i], acc[i][j]);
         else
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fr[buf][i], fr[buf][FM + j], acc[i][j], 0, 0, 0);
+            acc[i][j] = mfma16(fr[buf][i], fr[buf][FM + j], acc[i][j]);
     };
 
     const int nk = g.kdim / 64;
@@ -468,14 +476,15 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     else epilogue<BM, BN, WGM, WGN, EPI, false>(g, tc, acc, smem);
 }
 
-// Fragments (i, j) of wave `wave` of a WGM x WGN wave grid that lie entirely below the diagonal of a diagonal tile.
+// 16x16 fragments (i, j) of wave `wave` of a WGM x WGN wave grid whose enclosing 32x32 block lies entirely below
+// the diagonal of a diagonal tile (the epilogue masks at that granularity).
 template <int WTM, int WTN, int FM, int FN, int WGN>
 constexpr unsigned pp_skip_mask(int wave) {
     const int wm = wave / WGN, wn = wave % WGN;
     unsigned m = 0;
     for (int i = 0; i < FM; ++i)
         for (int j = 0; j < FN; ++j)
-            if (wm * WTM + i * 32 >= wn * WTN + j * 32 + 32) m |= 1u << (i * FN + j);
+            if ((wm * WTM + i * 16) / 32 > (wn * WTN + j * 16) / 32) m |= 1u << (i * FN + j);
     return m;
 }
 template <int WTM, int WTN, int FM, int FN, int WGN>
@@ -501,10 +510,11 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     constexpr int NW = WGM * WGN;
     constexpr int BK4 = 32, ROWB = 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
-    constexpr int FM = WTM / 32, FN = WTN / 32;
+    constexpr int FM = WTM / 16, FN = WTN / 16;
     constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
     constexpr int LA = BM / 16 / NW, LB = BN / 16 / NW;
     constexpr int NLD = LA + LB;
+    static_assert(FM * FN <= 32, "one mask bit per fragment");
     static_assert(NW == 8, "two groups of four waves, one of each per SIMD");
     static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "dma split");
     static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
@@ -528,11 +538,13 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
 #pragma unroll
     for (int n = 0; n < LA; ++n) offa[n] = (unsigned)(((wave * 16 * LA + n * 16 + drow) * BLK_COLS + dch) * 2);
     // BX: a k-tile of Q is BN/32 pieces of 32 rows x 32 columns, each a contiguous 2 KB run of one block; load
-    // instruction t of the tile (1 KB) is the half t%2 of piece t/2, in lane order
+    // instruction t of the tile (1 KB) is the half t%2 of piece t/2, in lane order, with the two 32-byte halves
+    // of a row swapped in rows whose k has bit 3 set (see qt_lane_offset)
+    const int qch = ((lane & 3) ^ (((drow >> 3) & 1) << 1)) * 8;
 #pragma unroll
     for (int n = 0; n < LB; ++n) {
         const int t = wave * LB + n;
-        offb[n] = QT ? (unsigned)(((t >> 1) * BLK_ELEMS + ((t & 1) * 16 + drow) * BLK_COLS + (lane & 3) * 8) * 2)
+        offb[n] = QT ? (unsigned)(((t >> 1) * BLK_ELEMS + ((t & 1) * 16 + drow) * BLK_COLS + qch) * 2)
                      : (unsigned)(((wave * 16 * LB + n * 16 + drow) * BLK_COLS + dch) * 2);
     }
     const int lds_a = wave * 16 * LA * ROWB;
@@ -560,21 +572,24 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
         for (int n = 0; n < LB; ++n) dma(bb, offb[n], st + lds_b + n * 16 * ROWB);
     };
 
-    f32x16 acc[FM][FN];
+    f32x4 acc[FM][FN];
 #pragma unroll
     for (int i = 0; i < FM; ++i)
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+            for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
     // Diagonal tile of a symmetric product: a fragment of a wave that lies entirely below the diagonal is the
     // mirror image of one another wave computes, and the epilogue does not read it.  Bit i*FN+j of a wave's mask:
     // skip that fragment's MFMAs (and the fragment reads nobody needs).
     const bool diag = EPI != EPI_BX && tc.ti == tc.tj;
-    const int sw = (lane >> 2) & 3, hi = lane >> 5;
-    const int a_off = (wm * WTM + (lane & 31)) * ROWB;
-    const int b_off = A_BYTES + (wn * WTN + (lane & 31)) * ROWB;
+    // fragment reads: lane l takes row l%16 of the fragment and the 16-byte chunk l/16 of its 64-byte row
+    // (chunk c of row r sits at c ^ ((r>>2)&3))
+    const int sw = (lane >> 2) & 3, kq = lane >> 4;
+    const int co = (kq ^ sw) << 4;
+    const int a_off = (wm * WTM + (lane & 15)) * ROWB + co;
+    const int b_off = A_BYTES + (wn * WTN + (lane & 15)) * ROWB + co;
 
     issue_tile(0);
     issue_tile(1);
@@ -584,45 +599,40 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     asm volatile("" ::: "memory");
     if (grp) __builtin_amdgcn_s_barrier();
 
-    // LDS read addresses: one register per operand, k-step and pair of stages; the stage inside
-    // the pair and the fragment index are instruction offsets (below 64 KB) once the k loop is
-    // unrolled by the four stages.
-    const unsigned char* ra[2][2];
+    // LDS read addresses: one register per operand (BX: per half of a piece) and pair of stages; the stage
+    // inside the pair and the fragment index are instruction offsets (below 64 KB) once the k loop is unrolled
+    // by the four stages.
+    const unsigned char* ra[2];
     const unsigned char* rb[2][2];
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-        const int co = (((ks << 1) | hi) ^ sw) << 4;
+    for (int half = 0; half < 2; ++half) {
+        ra[half] = smem + half * 2 * STAGE + a_off;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            ra[ks][half] = smem + half * 2 * STAGE + a_off + co;
-            rb[ks][half] = QT ? smem + half * 2 * STAGE + A_BYTES + (wn * WTN / 32) * 2048 + ks * 16 * 64 + qt_lane_offset(lane)
-                              : smem + half * 2 * STAGE + b_off + co;
-        }
+        for (int h = 0; h < 2; ++h)
+            rb[half][h] = QT ? smem + half * 2 * STAGE + A_BYTES + (wn * WTN / 32) * 2048 + qt_lane_offset(lane, h)
+                             : smem + half * 2 * STAGE + b_off;
     }
     auto body = [&](int kt, auto stage_c, auto mask_c) {
         constexpr int SIDX = decltype(stage_c)::value;
         constexpr unsigned MASK = decltype(mask_c)::value;
         auto kept = [](int i, int j) { return !((MASK >> (i * FN + j)) & 1); };
         // ---- M(kt)
-        bf16x8 fa[2][FM], fb[2][FN];
+        bf16x8 fa[FM], fb[FN];
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        for (int i = 0; i < FM; ++i) {
+            bool used = false;
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                bool used = false;
+            for (int j = 0; j < FN; ++j) used |= kept(i, j);
+            if (used) fa[i] = *(const bf16x8*)(ra[SIDX >> 1] + (SIDX & 1) * STAGE + i * 16 * ROWB);
+        }
 #pragma unroll
-                for (int j = 0; j < FN; ++j) used |= kept(i, j);
-                if (used) fa[ks][i] = *(const bf16x8*)(ra[ks][SIDX >> 1] + (SIDX & 1) * STAGE + i * 32 * ROWB);
-            }
+        for (int j = 0; j < FN; ++j) {
+            bool used = false;
 #pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                bool used = false;
-#pragma unroll
-                for (int i = 0; i < FM; ++i) used |= kept(i, j);
-                if (!used) continue;
-                if (QT) fb[ks][j] = lds_read_qt(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 2048);
-                else fb[ks][j] = *(const bf16x8*)(rb[ks][SIDX >> 1] + (SIDX & 1) * STAGE + j * 32 * ROWB);
-            }
+            for (int i = 0; i < FM; ++i) used |= kept(i, j);
+            if (!used) continue;
+            if (QT) fb[j] = lds_read_qt(rb[SIDX >> 1][j & 1] + (SIDX & 1) * STAGE + (j >> 1) * 2048);
+            else fb[j] = *(const bf16x8*)(rb[SIDX >> 1][0] + (SIDX & 1) * STAGE + j * 16 * ROWB);
         }
         issue_tile(kt + 3);
         WAIT_LGKM0();
@@ -634,16 +644,14 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
         __builtin_amdgcn_sched_barrier(0);
         // ---- C(kt)
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
+        for (int i = 0; i < FM; ++i)
 #pragma unroll
-            for (int i = 0; i < FM; ++i)
-#pragma unroll
-                for (int j = 0; j < FN; ++j) {
-                    if (QT)  // operands swapped: a lane then holds 4 consecutive columns of one row of the tile
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
-                    else if (kept(i, j))
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fb[ks][j], acc[i][j], 0, 0, 0);
-                }
+            for (int j = 0; j < FN; ++j) {
+                if (QT)  // operands swapped: a lane then holds 4 consecutive columns of one row of the tile
+                    acc[i][j] = mfma16(fb[j], fa[i], acc[i][j]);
+                else if (kept(i, j))
+                    acc[i][j] = mfma16(fa[i], fb[j], acc[i][j]);
+            }
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
@@ -736,6 +744,7 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
         case GEMM_CFG_128_PIPE: return launch_one<128, 128, 2, 2, EPI, 0>(g, nblocks, stream);
         case GEMM_CFG_256_PIPE: return launch_one<256, 256, 2, 4, EPI, 0>(g, nblocks, stream);
         case GEMM_CFG_256_PINGPONG: return launch_one<256, 256, 2, 4, EPI, 1>(g, nblocks, stream);
+        case GEMM_CFG_256_PIPE4W: return launch_one<256, 256, 2, 2, EPI, 0>(g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -746,7 +755,8 @@ int gemm_cfg_tile(int cfg) {
     switch (cfg) {
         case GEMM_CFG_128_PIPE: return 128;
         case GEMM_CFG_256_PIPE:
-        case GEMM_CFG_256_PINGPONG: return 256;
+        case GEMM_CFG_256_PINGPONG:
+        case GEMM_CFG_256_PIPE4W: return 256;
         default: return 0;
     }
 }

@@ -90,14 +90,14 @@ struct AdamConst {
 template <typename T>
 __device__ __forceinline__ void adam_one(float& p, float g, float& e1, float& e2, const AdamConst& am, float r1, float r2) {
     const float a = Mt<T>::rnd(lerp_aten(e1, g, am.w1, am.w1m1, am.small1));
-    const float g2 = Mt<T>::rnd(g * g);
+    const float g2 = materialized(Mt<T>::rnd(g * g));  // grad.square() is a tensor of its own
     const float bb = Mt<T>::rnd(lerp_aten(e2, g2, am.w2, am.w2m1, am.small2));
     e1 = a;
     e2 = bb;
     // a tensor divided by a python scalar is a multiplication by the scalar's fp32 reciprocal on a GPU
     const float ac = Mt<T>::rnd(a * r1);
     const float bc = Mt<T>::rnd(bb * r2);
-    const float den = Mt<T>::rnd(Mt<T>::rnd(__fsqrt_rn(bc)) + am.eps);
+    const float den = Mt<T>::rnd(Mt<T>::rnd(sqrtf(bc)) + am.eps);
     const float upd = Mt<T>::rnd(__fdiv_rn(ac, den));
     const float pd = Mt<T>::rnd(p * am.decay);
     p = fmaf(am.alpha, upd, pd);  // stored through Mt<T>::store*, which rounds
@@ -177,7 +177,7 @@ tensor_norm_kernel(const float* partials, const long* chunk_start, int dtype, fl
     float ss = 0.f;
     for (long c = chunk_start[t] + threadIdx.x; c < chunk_start[t + 1]; c += 256) ss += partials[c];
     ss = block_sum_256(ss, red);
-    if (threadIdx.x == 0) norms[t] = rnd_dtype(__fsqrt_rn(ss), dtype);
+    if (threadIdx.x == 0) norms[t] = rnd_dtype(sqrtf(ss), dtype);
 }
 
 // One block: norm of the per-tensor norms, rounded to the result dtype; written as fp32 (for the
@@ -189,7 +189,7 @@ total_norm_kernel(const float* norms, int n, int dtype, float* total_f32, void* 
     for (int t = threadIdx.x; t < n; t += 256) ss = fmaf(norms[t], norms[t], ss);
     ss = block_sum_256(ss, red);
     if (threadIdx.x == 0) {
-        const float tn = rnd_dtype(__fsqrt_rn(ss), dtype);
+        const float tn = rnd_dtype(sqrtf(ss), dtype);
         *total_f32 = tn;
         if (dtype == MUON_HIP_BF16) *(bf16_t*)total_typed = f2bf(tn);
         else *(float*)total_typed = tn;

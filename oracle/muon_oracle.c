@@ -180,7 +180,8 @@ void orc_adamw_f32(float* p, const float* g, float* e1, float* e2, size_t n, int
         float b = (fabsf(w2) < 0.5f) ? fmaf(w2, g2 - e2[i], e2[i]) : fmaf(w2 - 1.0f, g2 - e2[i], g2);
         e1[i] = a;
         e2[i] = b;
-        float upd = (a / c1) / (sqrtf(b / c2) + eps);
+        /* tensor / python scalar on a GPU: a multiplication by the scalar's fp32 reciprocal */
+        float upd = (a * (1.0f / c1)) / (sqrtf(b * (1.0f / c2)) + eps);
         float pv = p[i] * decay;
         p[i] = pv + alpha * upd;
     }

@@ -24,3 +24,13 @@ def oracle_c():
         subprocess.check_call(["make", "-C", odir])
     lib = ctypes.CDLL(so)
     return lib
+
+
+def pytest_terminal_summary(terminalreporter):
+    """Parity figures the GPU tests measured (worst relative errors against the oracle), also in quiet runs."""
+    from tests.helpers import PARITY_REPORT
+
+    if PARITY_REPORT:
+        terminalreporter.write_sep("-", "measured parity figures")
+        for line in PARITY_REPORT:
+            terminalreporter.write_line(line)

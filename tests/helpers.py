@@ -48,3 +48,13 @@ def c_newton_schulz(lib, G: torch.Tensor, steps: int) -> torch.Tensor:
     lib.orc_newton_schulz(Gc.ctypes.data_as(ctypes.c_void_p), rows, cols, steps, ctypes.c_double(3.4445),
                           ctypes.c_double(-4.7750), ctypes.c_double(2.0315), out.ctypes.data_as(ctypes.c_void_p))
     return bf16_from_u16(out)
+
+
+PARITY_REPORT = []
+
+
+def report_parity(line: str) -> None:
+    """Print a measured parity figure now and keep it for the end-of-run summary (tests/conftest.py), so that it
+    shows in the output of a quiet run, where the stdout of passing tests is dropped."""
+    print(line, flush=True)
+    PARITY_REPORT.append(line)

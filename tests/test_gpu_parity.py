@@ -11,7 +11,7 @@ import ctypes
 import pytest
 import torch
 
-from tests.helpers import MUON_HP, NAMES, QWEN25_05B, make_param_set, rel_fro
+from tests.helpers import MUON_HP, NAMES, QWEN25_05B, make_param_set, rel_fro, report_parity
 
 pytestmark = pytest.mark.gpu
 
@@ -227,7 +227,7 @@ def test_newton_schulz_config1(env):
     ref = O.newton_schulz(G, 5)
     got = mu.fast_newtonschulz(G.to(env["dev"]), 5)
     err = rel_fro(got, ref)
-    print("config1 rel fro", err, flush=True)
+    report_parity(f"config 1 (896x4864 fp32, seed 0, 5 iterations): NS-output error {err:.3e} (bound {NS_TOL})")
     assert err <= NS_TOL
     got_t = mu.fast_newtonschulz(G.mT.contiguous().to(env["dev"]), 5)
     assert rel_fro(got_t, O.newton_schulz(G.mT.contiguous(), 5)) <= NS_TOL
@@ -308,6 +308,25 @@ def test_momentum_stage(env, gdt, mdt, nesterov, shape):
         assert rel_fro(u.float(), u_ref.float()) <= 4e-3  # u is stored in the grad's bf16
 
 
+def _ns_via_stages(env, grads, moms, beta=0.95, nesterov=True, steps=5):
+    """The unscaled Newton-Schulz output of a bucket, read from the workspace: muon_hip_momentum_norm ->
+    muon_hip_ns_grouped -> muon_hip_ns_output on device tensors `grads` and `moms` (same shape; the momentum
+    buffers move in place).  Returns a dense bf16 [batch, rows, cols] tensor."""
+    lib, abi, dev = env["lib"], env["abi"], env["dev"]
+    rows, cols = grads[0].shape
+    nb = len(grads)
+    ws = torch.empty(abi.workspace_bytes(rows, cols, nb), dtype=torch.uint8, device=dev)
+    table = torch.tensor([t.data_ptr() for t in list(grads) + list(moms)], dtype=torch.int64, device=dev)
+    out = torch.full((nb, rows, cols), float("nan"), dtype=torch.bfloat16, device=dev)
+    a, b, c = env["O"].NS_COEFFS
+    abi.check(lib.muon_hip_momentum_norm(table.data_ptr(), table.data_ptr() + 8 * nb, abi.dtype_code(grads[0].dtype),
+                                         abi.dtype_code(moms[0].dtype), ws.data_ptr(), rows, cols, nb, beta, int(nesterov), 0, 0))
+    abi.check(lib.muon_hip_ns_grouped(ws.data_ptr(), rows, cols, nb, steps, a, b, c, 0))
+    abi.check(lib.muon_hip_ns_output(ws.data_ptr(), rows, cols, nb, steps, out.data_ptr(), 0))
+    torch.cuda.synchronize()
+    return out
+
+
 def _build_opts(env, weights, hp, dtype, momentum_dtype=None, adam=None):
     """GPU optimizer from this package and the CPU oracle on copies of the same tensors."""
     mu, O = env["mu"], env["O"]
@@ -330,12 +349,30 @@ def _build_opts(env, weights, hp, dtype, momentum_dtype=None, adam=None):
     return opt, orc, gp, cp
 
 
-def _check_step(opt, orc, gp, cp, grads, dtype, p_tol):
+def _check_step(opt, orc, gp, cp, grads, dtype, p_tol, env=None):
+    """One step on both sides; returns the worst update / momentum / parameter error.  The update error of an
+    fp32 parameter is recovered from the parameter delta.  A bf16 parameter's delta is mostly its own rounding,
+    so there the orthogonalised update is read directly: the stage entry points run on copies of the same
+    gradient and momentum before the optimizer steps (pass `env`)."""
     dev = gp[0].device
     for p, c, g in zip(gp, cp, grads):
         p.grad = g.clone().to(dtype).to(dev)
         c.grad = g.clone().to(dtype)
     before = [p.detach().clone() for p in gp]
+    staged = {}
+    if dtype != torch.float32:
+        assert env is not None
+        for gi, group in enumerate(opt.param_groups):
+            if not group["use_muon"]:
+                continue
+            for p in group["params"]:
+                st = opt.state.get(p, {})
+                m0 = st["momentum_buffer"].clone() if "momentum_buffer" in st else torch.zeros_like(
+                    p, dtype=opt.momentum_dtype or p.dtype)
+                o = _ns_via_stages(env, [p.grad.clone()], [m0], beta=group["momentum"], nesterov=group["nesterov"],
+                                   steps=group["ns_steps"])[0]
+                sc = env["mu"].scale_factor(p.shape[0], p.shape[1], group["rms_scale"])
+                staged[p] = (o.float() * env["O"]._f32(sc)).bfloat16()
     opt.step()
     orc.step()
     torch.cuda.synchronize()
@@ -356,6 +393,8 @@ def _check_step(opt, orc, gp, cp, grads, dtype, p_tol):
             o_gpu = (before[idx].double().cpu() * (1 - lr * wd) - p.detach().double().cpu()) / lr
             if dtype == torch.float32:
                 worst_u = max(worst_u, rel_fro(o_gpu, o_cpu))
+            else:
+                worst_u = max(worst_u, rel_fro(staged[p], o_cpu))
             worst_p = max(worst_p, rel_fro(p.detach(), c.detach()))
     return worst_u, worst_m, worst_p
 
@@ -373,7 +412,7 @@ def test_full_step_small_param_set_three_steps(env):
             g = torch.randn(*c.shape, generator=torch.Generator().manual_seed(100 + step))
             p.grad, c.grad = g.to(env["dev"]), g.clone()
         wu, wm, wp = _check_step(opt, orc, gp, cp, grads[step], torch.float32, None)
-        print(f"step {step}: update {wu:.3e} momentum {wm:.3e} param {wp:.3e}", flush=True)
+        report_parity(f"config 2 slice (2 layers, fp32) step {step}: update {wu:.3e} momentum {wm:.3e} param {wp:.3e}")
         assert wu <= NS_TOL and wm <= MOM_TOL
         assert wp <= 2e-3  # params move by lr*update each step; 2e-2 of that, relative to ||p||
         for ai, (p, c) in enumerate(zip(ga, ca)):
@@ -389,8 +428,9 @@ def test_full_step_bf16_params(env, momentum_dtype):
     weights, grads = make_param_set(spec, layers=2, seed=11, steps=2, dtype=torch.bfloat16)
     opt, orc, gp, cp = _build_opts(env, weights, MUON_HP, torch.bfloat16, momentum_dtype=momentum_dtype)
     for step in range(2):
-        wu, wm, wp = _check_step(opt, orc, gp, cp, grads[step], torch.bfloat16, None)
-        print(f"bf16 step {step}: momentum {wm:.3e} param {wp:.3e}", flush=True)
+        wu, wm, wp = _check_step(opt, orc, gp, cp, grads[step], torch.bfloat16, None, env=env)
+        report_parity(f"bf16 params (momentum {momentum_dtype}) step {step}: update {wu:.3e} momentum {wm:.3e} param {wp:.3e}")
+        assert wu <= NS_TOL
         assert wm <= (MOM_TOL if momentum_dtype == torch.float32 else 1e-3)
         assert wp <= 4e-3  # a few bf16 roundings of p differ where the update differs
 
@@ -406,11 +446,11 @@ def test_full_step_ragged_and_tall_shapes(env, dtype):
     opt, orc, gp, cp = _build_opts(env, weights, MUON_HP, dtype, momentum_dtype=torch.float32 if dtype == torch.bfloat16 else None)
     for step in range(2):
         grads = [1e-3 * torch.randn(*s, generator=gen) for s in shapes]
-        wu, wm, wp = _check_step(opt, orc, gp, cp, grads, dtype, None)
+        wu, wm, wp = _check_step(opt, orc, gp, cp, grads, dtype, None, env=env)
         print(f"ragged {dtype} step {step}: update {wu:.3e} momentum {wm:.3e} param {wp:.3e}", flush=True)
-        assert wm <= MOM_TOL
+        assert wm <= MOM_TOL and wu <= NS_TOL
         if dtype == torch.float32:
-            assert wu <= NS_TOL and wp <= 2e-3  # params move by lr*update; 2e-2 of that relative to ||p||
+            assert wp <= 2e-3  # params move by lr*update; 2e-2 of that relative to ||p||
         else:
             assert wp <= 4e-3
 
@@ -435,6 +475,147 @@ def test_grouped_equals_per_matrix_bitwise(env):
     torch.cuda.synchronize()
     for p, q in zip(pa, pb):
         assert torch.equal(p.detach(), q.detach())
+
+
+def test_grouped_equals_per_matrix_bitwise_on_256_tiles(env):
+    """The same for shapes whose short side is a whole number of 256-tiles (ping-pong and split-tail kernels) and
+    for the expert shapes 768x2048 / 2048x768 (128-tiles): bf16 parameters, fp32 momentum, three matrices per
+    bucket against three launches of one."""
+    mu, dev = env["mu"], env["dev"]
+    spec = dict(q=(512, 512), k=(768, 2048), v=(768, 2048), o=(512, 512), gate=(2048, 768), up=(1024, 512), down=(512, 1024))
+    weights, grads = make_param_set(spec, layers=3, seed=15, steps=1, dtype=torch.bfloat16)
+    pa = [torch.nn.Parameter(w.clone().to(dev)) for _, w in weights]
+    pb = [torch.nn.Parameter(w.clone().to(dev)) for _, w in weights]
+    for p, q, g in zip(pa, pb, grads[0]):
+        p.grad, q.grad = g.to(dev), g.to(dev)
+    opt = mu.Muon([dict(params=pa, use_muon=True, **MUON_HP)], momentum_dtype=torch.float32)
+    opt.step()
+    group = dict(opt.param_groups[0])
+    for q in pb:
+        st = {"momentum_buffer": torch.zeros_like(q, dtype=torch.float32)}
+        w = mu.SingelDeviceWork(q, st, group, 0)
+        w.start()
+        w.finish()
+    torch.cuda.synchronize()
+    for (name, _), p, q in zip(weights, pa, pb):
+        assert torch.equal(p.detach(), q.detach()), name
+
+
+BUCKET_SHAPES = [(4096, 4096), (1024, 4096), (12288, 4096), (4096, 12288),      # Qwen3-8B (benchmark config 3)
+                 (768, 2048), (2048, 768), (512, 2048), (4096, 2048), (2048, 4096)]  # Qwen3-MoE-30B-A3B (config 5)
+
+
+@pytest.mark.parametrize("rows,cols", BUCKET_SHAPES)
+def test_bucket_shapes_grouped_ns_output_within_bound(env, rows, cols):
+    """Every bucket shape of the two bf16 benchmark configurations in a grouped launch (bf16 gradients, fp32
+    momentum, several matrices): the orthogonalised update itself, read from the workspace after
+    muon_hip_momentum_norm -> muon_hip_ns_grouped -> muon_hip_ns_output, per matrix within 2e-2 relative
+    Frobenius error of (a) fast_newtonschulz's own torch expressions (muon_utils.py:138-156) evaluated on the
+    device for every matrix, with torch's fp32-accumulated product standing in for the Triton kernel, and (b) the
+    CPU oracle for the first matrix."""
+    O, dev = env["O"], env["dev"]
+    batch = 6 if rows * cols <= 2048 * 2048 else 2
+    print(f"bucket {rows}x{cols} batch={batch}", flush=True)
+    gen = torch.Generator().manual_seed(rows * 3 + cols)
+    g = [(1e-3 * torch.randn(rows, cols, generator=gen)).bfloat16() for _ in range(batch)]
+    m = [1e-3 * torch.randn(rows, cols, generator=gen) for _ in range(batch)]
+    gd, md = [t.to(dev) for t in g], [t.to(dev) for t in m]
+    m_ref = [t.clone() for t in md]
+    out = _ns_via_stages(env, gd, md)
+    assert torch.isfinite(out).all()
+    torch.set_num_threads(16)
+    worst = 0.0
+    for i in range(batch):
+        # the blend the extension defines for (bf16 g, fp32 m): gradient upcast, fp32 lerps
+        gf = gd[i].float()
+        m_ref[i].lerp_(gf, 1 - 0.95)
+        u = gf.lerp_(m_ref[i], 0.95)
+        assert torch.equal(md[i], m_ref[i]), "fp32 momentum is the device lerp, bit for bit"
+        ref_dev = O.newton_schulz(u, 5, literal=True)
+        e_dev = rel_fro(out[i], ref_dev)
+        line = f"  matrix {i}: vs torch on device {e_dev:.3e}"
+        assert e_dev <= NS_TOL, (rows, cols, i, e_dev)
+        worst = max(worst, e_dev)
+        if i == 0:
+            e_cpu = rel_fro(out[i], O.newton_schulz(u.cpu(), 5))
+            line += f", vs CPU oracle {e_cpu:.3e}"
+            assert e_cpu <= NS_TOL, (rows, cols, e_cpu)
+            worst = max(worst, e_cpu)
+        print(line, flush=True)
+    report_parity(f"bucket {rows}x{cols} x{batch} grouped (bf16 g, fp32 m): worst NS-output error {worst:.3e} (bound {NS_TOL})")
+
+
+def test_module_substitution_factory_groups_and_checkpoint_round_trip(env, tmp_path, monkeypatch):
+    """The integration recipe end to end: the module installed as lmms_engine.utils.muon_utils, the optimizer
+    built through that import from the four groups Trainer.create_optimizer makes (train/hf/trainer.py:417-465),
+    stepped on the GPU, and its state_dict sent through torch.save / torch.load (weights only, as a checkpoint
+    is read back) into a fresh optimizer that then continues bit-identically, fp32 momentum included."""
+    import sys
+    import types
+
+    mu, dev = env["mu"], env["dev"]
+    pkg, sub = types.ModuleType("lmms_engine"), types.ModuleType("lmms_engine.utils")
+    pkg.utils, sub.muon_utils = sub, mu
+    monkeypatch.setitem(sys.modules, "lmms_engine", pkg)
+    monkeypatch.setitem(sys.modules, "lmms_engine.utils", sub)
+    monkeypatch.setitem(sys.modules, "lmms_engine.utils.muon_utils", mu)
+    from lmms_engine.utils.muon_utils import Muon
+
+    assert Muon is mu.Muon
+
+    def model(seed):
+        gen = torch.Generator().manual_seed(seed)
+        mk = lambda *s: torch.nn.Parameter((0.02 * torch.randn(*s, generator=gen)).bfloat16().to(dev))
+        return dict(q=mk(256, 256), up=mk(640, 256), down=mk(256, 640), emb=mk(1000, 64), norm=mk(256))
+
+    def factory(ps, **extra):
+        lr = 1e-3
+        groups = [
+            dict(params=[ps["q"]], use_muon=True, lr=lr, momentum=0.95, weight_decay=0.01),
+            dict(params=[ps["up"], ps["down"]], use_muon=True, lr=lr, momentum=0.95, weight_decay=0.0),
+            dict(params=[ps["emb"]], use_muon=False, lr=lr, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01),
+            dict(params=[ps["norm"]], use_muon=False, lr=lr, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.0),
+        ]
+        return Muon(groups, defaults=dict(lr=lr), is_deepspeed_enabled=False, **extra)
+
+    def set_grads(ps, seed):
+        gen = torch.Generator().manual_seed(seed)
+        for p in ps.values():
+            p.grad = (1e-3 * torch.randn(*p.shape, generator=gen)).bfloat16().to(dev)
+
+    ps = model(1)
+    opt = factory(ps, momentum_dtype=torch.float32)
+    for step in range(2):
+        set_grads(ps, 10 + step)
+        opt.step()
+    path = tmp_path / "optimizer.pt"
+    torch.save(opt.state_dict(), path)
+    sd = torch.load(path, map_location=dev, weights_only=True)
+    assert sd["state"][0]["momentum_buffer"].dtype == torch.float32
+    assert sd["state"][3]["step"] == 2 and set(sd["state"][3]) == {"exp_avg", "exp_avg_sq", "step"}
+    ps2 = {k: torch.nn.Parameter(v.detach().clone()) for k, v in ps.items()}
+    opt2 = factory(ps2, momentum_dtype=torch.float32)
+    opt2.load_state_dict(sd)
+    for p, q in zip(ps.values(), ps2.values()):
+        if p.ndim == 2 and p is not ps["emb"]:
+            assert opt2.state[q]["momentum_buffer"].dtype == torch.float32
+            assert torch.equal(opt2.state[q]["momentum_buffer"], opt.state[p]["momentum_buffer"])
+    set_grads(ps, 99)
+    set_grads(ps2, 99)
+    opt.step()
+    opt2.step()
+    torch.cuda.synchronize()
+    for k in ps:
+        assert torch.equal(ps[k].detach(), ps2[k].detach()), k
+    # releasing the workspace between steps changes nothing but the memory held
+    opt.release_workspace()
+    assert opt._workspaces == {}
+    set_grads(ps, 100)
+    set_grads(ps2, 100)
+    opt.step()
+    opt2.step()
+    for k in ps:
+        assert torch.equal(ps[k].detach(), ps2[k].detach()), k
 
 
 def test_reference_bug_compat_and_rms_scale(env):
@@ -612,7 +793,7 @@ def test_full_size_newton_schulz(env, rows, cols):
     torch.set_num_threads(16)
     ref = O.newton_schulz(G, 5)
     err = rel_fro(out, ref)
-    print(f"  vs oracle {err:.3e}", flush=True)
+    report_parity(f"full-size NS {rows}x{cols} (N(0,1), seed 2): error vs oracle {err:.3e} (bound {NS_TOL})")
     assert err <= NS_TOL
 
 
