@@ -435,7 +435,8 @@ struct AdamMath {
 };
 
 // adam_update (muon_utils.py:178-183) for one element, every in-place op rounded in the tensor dtype.  A tensor
-// divided by a python scalar is evaluated on a GPU as a multiplication by the scalar's fp32 reciprocal.
+// divided by a python scalar is evaluated on a GPU as a multiplication by the scalar's reciprocal (computed in
+// double precision, narrowed to fp32).
 template <typename T>
 __device__ __forceinline__ float adam_moments(float gi, float& e1, float& e2, const AdamMath& am) {
     const float a = Ld<T>::rnd(lerp_aten(e1, gi, am.w1, am.w1m1, am.small1));
@@ -636,8 +637,9 @@ AdamMath adam_math(int step, double lr, double b1, double b2, double eps, double
     AdamMath am;
     lerp_consts(1.0 - b1, am.w1, am.w1m1, am.small1);
     lerp_consts(1.0 - b2, am.w2, am.w2m1, am.small2);
-    am.r1 = 1.0f / (float)(1.0 - pow(b1, (double)step));
-    am.r2 = 1.0f / (float)(1.0 - pow(b2, (double)step));
+    // the reciprocal is taken in double precision and then narrowed, as ATen does for a python-scalar divisor
+    am.r1 = (float)(1.0 / (1.0 - pow(b1, (double)step)));
+    am.r2 = (float)(1.0 / (1.0 - pow(b2, (double)step)));
     am.eps = (float)eps;
     am.decay = (float)(1.0 - lr * wd);
     am.alpha = (float)(-lr);

@@ -94,7 +94,7 @@ __device__ __forceinline__ void adam_one(float& p, float g, float& e1, float& e2
     const float bb = Mt<T>::rnd(lerp_aten(e2, g2, am.w2, am.w2m1, am.small2));
     e1 = a;
     e2 = bb;
-    // a tensor divided by a python scalar is a multiplication by the scalar's fp32 reciprocal on a GPU
+    // a tensor divided by a python scalar is a multiplication by the scalar's reciprocal on a GPU
     const float ac = Mt<T>::rnd(a * r1);
     const float bc = Mt<T>::rnd(bb * r2);
     const float den = Mt<T>::rnd(Mt<T>::rnd(sqrtf(bc)) + am.eps);
@@ -113,7 +113,7 @@ adamw_multi_kernel(const void* const* p_ptrs, const void* const* g_ptrs, const v
     const T* g = (const T*)g_ptrs[r.t] + r.begin;
     T* e1 = (T*)e1_ptrs[r.t] + r.begin;
     T* e2 = (T*)e2_ptrs[r.t] + r.begin;
-    const float r1 = __fdiv_rn(1.0f, (float)bias1[r.t]), r2 = __fdiv_rn(1.0f, (float)bias2[r.t]);
+    const float r1 = (float)(1.0 / bias1[r.t]), r2 = (float)(1.0 / bias2[r.t]);  // double reciprocal, then narrowed
     const bool vec = ((((uintptr_t)p) | ((uintptr_t)g) | ((uintptr_t)e1) | ((uintptr_t)e2)) & 15) == 0;
     const long n8 = vec ? r.len / 8 : 0;
     for (long i = threadIdx.x; i < n8; i += 256) {

@@ -169,7 +169,8 @@ void orc_scale_update_bf16(uint16_t* p, uint16_t* O, size_t n, double scale_, do
 void orc_adamw_f32(float* p, const float* g, float* e1, float* e2, size_t n, int step, double lr_, double b1_,
                    double b2_, double eps_, double wd_) {
     const float w1 = (float)(1.0 - b1_), w2 = (float)(1.0 - b2_);
-    const float c1 = (float)(1.0 - pow(b1_, step)), c2 = (float)(1.0 - pow(b2_, step));
+    /* tensor / python scalar on a GPU: a multiplication by the scalar's reciprocal, taken in double and narrowed */
+    const float r1 = (float)(1.0 / (1.0 - pow(b1_, step))), r2 = (float)(1.0 / (1.0 - pow(b2_, step)));
     const float eps = (float)eps_;
     const float decay = (float)(1.0 - lr_ * wd_);
     const float alpha = (float)(-lr_);
@@ -180,8 +181,7 @@ void orc_adamw_f32(float* p, const float* g, float* e1, float* e2, size_t n, int
         float b = (fabsf(w2) < 0.5f) ? fmaf(w2, g2 - e2[i], e2[i]) : fmaf(w2 - 1.0f, g2 - e2[i], g2);
         e1[i] = a;
         e2[i] = b;
-        /* tensor / python scalar on a GPU: a multiplication by the scalar's fp32 reciprocal */
-        float upd = (a * (1.0f / c1)) / (sqrtf(b * (1.0f / c2)) + eps);
+        float upd = (a * r1) / (sqrtf(b * r2) + eps);
         float pv = p[i] * decay;
         p[i] = pv + alpha * upd;
     }

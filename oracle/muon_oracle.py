@@ -197,8 +197,8 @@ def adam_update(grad: Tensor, buf1: Tensor, buf2: Tensor, step: int, betas, eps:
     """muon_utils.py:178-183.
 
     `literal=True` is the reference's text evaluated by torch on the CPU.  The default restates what the same
-    text computes on a GPU, where ATen evaluates tensor / python-scalar as tensor * (1.0f / scalar_f32) (its CPU
-    kernel divides); the two differ by at most one fp32 ulp before the rounding to the tensor dtype.  The GPU
+    text computes on a GPU, where ATen evaluates tensor / python-scalar as tensor * float(1.0 / scalar), the reciprocal
+    taken in double precision (its CPU kernel divides); the two differ by at most one fp32 ulp before the rounding to the tensor dtype.  The GPU
     form is pinned by a device-side test against torch itself (tests/test_gpu_torch_device.py).
     """
     buf1.lerp_(grad, 1 - betas[0])
@@ -207,9 +207,8 @@ def adam_update(grad: Tensor, buf1: Tensor, buf2: Tensor, step: int, betas, eps:
         buf1c = buf1 / (1 - betas[0] ** step)
         buf2c = buf2 / (1 - betas[1] ** step)
     else:
-        one = torch.tensor(1.0, dtype=torch.float32)
-        inv1 = one / torch.tensor(1 - betas[0] ** step, dtype=torch.float32)
-        inv2 = one / torch.tensor(1 - betas[1] ** step, dtype=torch.float32)
+        inv1 = torch.tensor(1.0 / (1 - betas[0] ** step), dtype=torch.float32)
+        inv2 = torch.tensor(1.0 / (1 - betas[1] ** step), dtype=torch.float32)
         buf1c = (buf1.float() * inv1).to(buf1.dtype)
         buf2c = (buf2.float() * inv2).to(buf2.dtype)
     return buf1c / (buf2c.sqrt() + eps)
