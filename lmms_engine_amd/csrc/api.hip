@@ -154,6 +154,13 @@ int check_gemm(int cfg, int Mp, int Kp, int batch, int& tile) {
     return 0;
 }
 
+#ifdef MUON_TILE_TRACE
+long* g_trace = nullptr;  // measurement builds only
+#define SET_TRACE(g) (g).trace = g_trace
+#else
+#define SET_TRACE(g) do { } while (0)
+#endif
+
 // The three products on blocked buffers; matrix b of a batch starts at b * blocked_elems(rows, cols).
 int do_syrk(int cfg, const bf16_t* X, bf16_t* A, int Mp, int Kp, int batch, hipStream_t s) {
     GemmArgs g = {};
@@ -167,6 +174,7 @@ int do_syrk(int cfg, const bf16_t* X, bf16_t* A, int Mp, int Kp, int batch, hipS
     g.C = g.Ct = A;
     g.strideC = g.strideCt = blocked_elems(Mp, Mp);
     g.cbC = g.cbCt = Mp / BLK_COLS;
+    SET_TRACE(g);
     Timed t(MUON_HIP_K_SYRK, s);
     hipError_t e = launch_gemm_nt(cfg, EPI_SYRK, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "syrk launch");
@@ -189,6 +197,7 @@ int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b,
     g.cbEt = Mp / BLK_COLS;
     g.s0 = (float)b;
     g.s1 = (float)c;
+    SET_TRACE(g);
     Timed t(MUON_HIP_K_SYMPOLY, s);
     hipError_t e = launch_gemm_nt(cfg, EPI_SYMPOLY, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "sympoly launch");
@@ -214,6 +223,7 @@ int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int K
     g.strideEt = blocked_elems(Mp, Kp);
     g.cbEt = Kp / BLK_COLS;
     g.s0 = (float)a;
+    SET_TRACE(g);
     Timed t(MUON_HIP_K_BX, s);
     hipError_t e = launch_gemm_nt(cfg, EPI_BX, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "bx launch");
@@ -224,6 +234,13 @@ int dtype_ok(int d) { return d == MUON_HIP_F32 || d == MUON_HIP_BF16; }
 }  // namespace
 
 extern "C" {
+
+#ifdef MUON_TILE_TRACE
+int muon_hip_debug_set_trace(void* buf) {
+    g_trace = (long*)buf;
+    return 0;
+}
+#endif
 
 int muon_hip_version(void) { return 100; }
 

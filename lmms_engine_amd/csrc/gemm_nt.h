@@ -8,8 +8,7 @@ enum {
     GEMM_CFG_128_PIPE = 0,      // 128x128 tile, 4 waves, 64-column k-tiles in two LDS stages
     GEMM_CFG_256_PIPE = 1,      // 256x256 tile, 8 waves, the same pipeline
     GEMM_CFG_256_PINGPONG = 2,  // 256x256 tile, 8 waves in two alternating groups, four stages of 32 columns
-    GEMM_CFG_256_PIPE4W = 3,    // 256x256 tile, 4 waves of 128x128 (one per SIMD), 64-column k-tiles in two stages
-    GEMM_CFG_COUNT = 4
+    GEMM_CFG_COUNT = 3
 };
 
 struct GemmArgs {
@@ -32,6 +31,9 @@ struct GemmArgs {
     int cbEt;
     float s0, s1;           // SYMPOLY: (b, c); BX: (a, -)
     int big_blocks;         // set by the launcher: workgroups that compute whole 256x256 tiles (split-tail kernel)
+#ifdef MUON_TILE_TRACE
+    long* trace;            // measurement builds only: 8 longs per workgroup
+#endif
 };
 
 constexpr int GEMM_CU_COUNT = 256;  // compute units of the part: one 256x256 workgroup each
