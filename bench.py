@@ -181,9 +181,10 @@ def extras(params, pd, dev, reps):
     return res
 
 
-def _event_ms(fn, reps, torch):
-    """Mean milliseconds of fn() over `reps` calls after one warm-up call, from events on the current stream."""
-    fn()
+def _event_ms(fn, reps, torch, warm=1):
+    """Mean milliseconds of fn() over `reps` calls after `warm` warm-up calls, from events on the current stream."""
+    for _ in range(warm):
+        fn()
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     a.record()
@@ -296,6 +297,34 @@ def operand_power(dev, M=4096, K=12288, nb=16, reps=10):
     return res
 
 
+def mfma_probe(dev, iters=40000, reps=25):
+    """Loops of nothing but MFMAs (muon_hip_mfma_probe): both instruction shapes, operands with random mantissas
+    and constant operands.  The sustained rate is what the part's power management leaves of the 2.5 PFLOP/s."""
+    import ctypes
+
+    import torch
+
+    from lmms_engine_amd import _abi
+
+    lib = _abi.lib()
+    n = _abi.PROBE_OPERAND_BYTES // 2
+    sink = torch.empty(_abi.PROBE_SINK_FLOATS, dtype=torch.float32, device=dev)
+    res = {}
+    for label in ("random", "constant"):
+        ops = (torch.randn(n, device=dev) * 0.02).bfloat16() if label == "random" else torch.full((n,), 0.0078125, dtype=torch.bfloat16, device=dev)
+        res[label] = {}
+        for shape, name in ((0, "v_mfma_f32_32x32x16_bf16"), (1, "v_mfma_f32_16x16x32_bf16")):
+            flop = ctypes.c_double()
+            fn = lambda: _abi.check(lib.muon_hip_mfma_probe(ops.data_ptr(), sink.data_ptr(), shape, iters, ctypes.byref(flop),
+                                                            _abi.stream_ptr(dev)))
+            # about half a second of back-to-back launches behind a warm-up of the same kind: the clock follows
+            # the power drawn over tens of milliseconds
+            ms = _event_ms(fn, reps, torch, warm=8)
+            res[label][name] = {"ms": ms, "tflops": flop.value / (ms * 1e-3) / 1e12}
+    res["what"] = f"{reps} launches of {iters} iterations each after 8 warm-up launches, per instruction and operand content"
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -343,7 +372,7 @@ def main():
     if args.gemm_config >= 0:
         _abi.check(_abi.lib().muon_hip_set_gemm_config(args.gemm_config), "set_gemm_config")
     if args.operand_power_only:
-        print(json.dumps({"operand_power": operand_power(dev)}))
+        print(json.dumps({"operand_power": operand_power(dev), "mfma_probe": mfma_probe(dev)}))
         return
     w = WORKLOADS[args.workload]
     layers = args.layers or w["layers"]
@@ -454,6 +483,7 @@ def main():
         out["extras"] = extras(params, pd, dev, args.steps)
     if args.operand_power:
         out["operand_power"] = operand_power(dev)
+        out["mfma_probe"] = mfma_probe(dev)
     if not args.no_gpu_oracle:
         moms = [opt.state[p]["momentum_buffer"] for p in params]
         out["gpu_oracle"] = gpu_oracle(params, moms, shapes, flops_step)

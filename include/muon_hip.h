@@ -223,6 +223,15 @@ int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long
  * of HIP events on its own stream; muon_hip_timing_read waits for them and returns the summed
  * duration and launch count of one kernel id since timing was enabled. */
 int muon_hip_timing_enable(int on);
+
+/* A loop of nothing but MFMAs, for measuring what the matrix pipes sustain under the part's power management.
+ * No counterpart in the reference.  shape 0: v_mfma_f32_32x32x16_bf16, shape 1: v_mfma_f32_16x16x32_bf16, on one
+ * workgroup of 8 waves per compute unit with the register footprint of the GEMM kernels.  `operands` holds
+ * MUON_HIP_PROBE_OPERAND_BYTES of bf16 values chosen by the caller (random, constant ...), `sink` receives
+ * MUON_HIP_PROBE_SINK_FLOATS floats; *flop is the work of the launch.  Time it with events on `stream`. */
+#define MUON_HIP_PROBE_OPERAND_BYTES (256L * 12 * 512 * 16)
+#define MUON_HIP_PROBE_SINK_FLOATS (256L * 512)
+int muon_hip_mfma_probe(const void* operands, void* sink, int shape, int iters, double* flop, void* stream);
 int muon_hip_timing_read(int kernel_id, double* total_ms, long* launches);
 
 #ifdef __cplusplus

@@ -22,6 +22,7 @@ KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "app
                 "grad_norm", "clip_scale"]
 MULTI_CHUNK = 16384  # MUON_HIP_MULTI_CHUNK
 STATIC_MAX_CHUNKS = 1 << 20  # MUON_HIP_STATIC_MAX_CHUNKS
+PROBE_OPERAND_BYTES, PROBE_SINK_FLOATS = 256 * 12 * 512 * 16, 256 * 512  # MUON_HIP_PROBE_*
 
 # name -> (restype, argtypes); mirrors include/muon_hip.h one to one
 SIGNATURES = {
@@ -59,6 +60,7 @@ SIGNATURES = {
     "muon_hip_total_norm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "muon_hip_clip_scale": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_int, c_double,
                                     c_void_p]),
+    "muon_hip_mfma_probe": (c_int, [c_void_p, c_void_p, c_int, c_int, POINTER(c_double), c_void_p]),
     "muon_hip_timing_enable": (c_int, [c_int]),
     "muon_hip_timing_read": (c_int, [c_int, POINTER(c_double), POINTER(c_long)]),
 }

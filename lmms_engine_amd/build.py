@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libmuon_hip.so")
-SOURCES = ["gemm_nt.hip", "elementwise.hip", "multi_tensor.hip", "api.hip"]
+SOURCES = ["gemm_nt.hip", "elementwise.hip", "multi_tensor.hip", "probe.hip", "api.hip"]
 # Packed-fp32 VALU forms stay off for every device function.
 HIP_FLAGS = [
     "--offload-arch=gfx950",

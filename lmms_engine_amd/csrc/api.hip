@@ -11,6 +11,7 @@
 #include "elementwise.h"
 #include "gemm_nt.h"
 #include "multi_tensor.h"
+#include "probe.h"
 
 namespace {
 
@@ -563,6 +564,14 @@ int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long
     const MultiTensorList l{g_ptrs, numel, chunk_start, n, chunks};
     hipError_t e = launch_clip_scale_multi(l, dtype, total_f32, norm_dtype, max_norm, s);
     return e == hipSuccess ? 0 : hip_fail(e, "clip_scale launch");
+}
+
+int muon_hip_mfma_probe(const void* operands, void* sink, int shape, int iters, double* flop, void* stream) {
+    if (!operands || !sink) return fail(MUON_HIP_EINVAL, "null buffer");
+    if ((shape != 0 && shape != 1) || iters <= 0) return fail(MUON_HIP_EINVAL, "shape is 0 or 1 and iters positive");
+    hipError_t e = launch_mfma_probe(operands, (float*)sink, shape, iters, (hipStream_t)stream);
+    if (flop) *flop = MUON_PROBE_FLOP_PER_ITER * iters;
+    return e == hipSuccess ? 0 : hip_fail(e, "mfma_probe launch");
 }
 
 int muon_hip_timing_enable(int on) {

@@ -1,11 +1,11 @@
 // GEMM family for the Newton-Schulz chain on gfx950, built on v_mfma_f32_16x16x32_bf16.
 //
 // Why the 16x16x32 instruction: under matrix-pipe load the part lowers its clock to stay inside its power
-// limit, and on operands with random mantissas a loop of nothing but 32x32x16 MFMAs sustains about 1.3 PFLOP/s
-// while the same loop of 16x16x32 MFMAs sustains about 2.05 (both reach 2.4 on constant operands): the deeper
-// dot product updates each fp32 accumulator half as often per FLOP.  Operand fragment: lane l holds row l%16,
-// eight consecutive k from 8*(l/16) (16 bytes).  Accumulator fragment: lane l holds column l%16, rows
-// 4*(l/16)+0..3 (f32x4).
+// limit, and on operands with random mantissas a loop of nothing but MFMAs (muon_hip_mfma_probe) sustains about
+// 1.85 PFLOP/s with 32x32x16 and about 2.09 with 16x16x32 (both reach 2.45 on constant operands): the deeper dot
+// product updates each fp32 accumulator half as often per FLOP.  The same kernels built on 32x32x16 ran 4 to 8 %
+// slower at a 3 to 9 % lower clock.  Operand fragment: lane l holds row l%16, eight consecutive k from 8*(l/16)
+// (16 bytes).  Accumulator fragment: lane l holds column l%16, rows 4*(l/16)+0..3 (f32x4).
 //
 // The three products of one NS iteration:
 //   SYRK     A  = bf(X Xt)                         P = Q = X   (M x K)           C[i][j] = sum_k P[i][k] Q[j][k]

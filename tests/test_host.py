@@ -304,3 +304,7 @@ def test_argument_errors_are_reported_before_any_launch():
     rejected(lib.muon_hip_clip_scale(tbl, tbl, tbl, 1, 1, F32, None, F32, 1.0, None), EINVAL, "null total")
     rejected(lib.muon_hip_clip_scale(tbl, tbl, tbl, 1, 1 << 31, F32, tbl, F32, 1.0, None), ESHAPE, "chunks exceed")
     rejected(lib.muon_hip_timing_read(99, None, None), EINVAL, "kernel id")
+    rejected(lib.muon_hip_mfma_probe(None, tbl, 0, 10, None, None), EINVAL, "null buffer")
+    rejected(lib.muon_hip_mfma_probe(tbl, tbl, 2, 10, None, None), EINVAL, "shape")
+    rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, (1 << 20) + 1, F32, tbl, None), ESHAPE, "built-in scratch")
+    rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, 1, F32, None, None), EINVAL, "null output")
