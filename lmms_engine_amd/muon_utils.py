@@ -246,6 +246,39 @@ def muon_update(grad, momentum, beta=0.95, ns_steps=5, nesterov=True, rms_scale=
 # --------------------------------------------------------------------------------------
 # grouped launcher
 # --------------------------------------------------------------------------------------
+_CU_COUNT = 256  # one 256x256 GEMM workgroup per compute unit and round
+
+
+def _pick_chunk(n: int, cap: int, rows: int, cols: int) -> int:
+    """Matrices per grouped launch for a bucket of n: about `cap` (what the workspace limit holds; up to an eighth
+    more when that lands on whole rounds), chosen so that the tile counts of the three products leave the last
+    round of the 256 compute units as full as possible.  A launch of t tiles runs ceil(t / 256) rounds (a last
+    round of at most 64 tiles is cut into quarter tiles and costs about 0.6 of a round) plus about a third of a
+    round of ramp-up and tail; a tile of X.Xt costs ~K, one of b.A + c.A.A and of a.X + B.X ~M."""
+    if cap >= n or cap <= 2:
+        return max(1, min(n, cap))
+    M, K = min(rows, cols), max(rows, cols)
+    if M % 256 or M < 512:
+        return cap  # 128-tiles: many small tiles, rounds hardly matter
+    T, TN = M // 256, -(-K // 256)
+    tri, rect = T * (T + 1) // 2, T * TN
+
+    def rounds(t):
+        full, rest = divmod(t, _CU_COUNT)
+        return full + (0.0 if rest == 0 else 0.6 if rest <= _CU_COUNT // 4 and full > 0 else 1.0)
+
+    def cost(nb):
+        return (rounds(tri * nb) + 0.35) * (K + M) + (rounds(rect * nb) + 0.35) * M
+
+    best, best_cost = cap, None
+    for nb in range(max(1, cap // 2), min(n, cap + cap // 8) + 1):
+        chunks, last = divmod(n, nb)
+        c = chunks * cost(nb) + (cost(last) if last else 0.0)
+        if best_cost is None or c < best_cost * (1 - 1e-9):
+            best, best_cost = nb, c
+    return best
+
+
 def _muon_bucket_step(params, grads, moms, group, ns_steps, nesterov, write_back_grad, ws_holder, ws_limit):
     """All stages of the Muon step for same-shape, same-dtype parameters on one device."""
     p0 = params[0]
@@ -257,7 +290,7 @@ def _muon_bucket_step(params, grads, moms, group, ns_steps, nesterov, write_back
     scale = scale_factor(rows, cols, group["rms_scale"])
     n = len(params)
     per = _abi.workspace_bytes(rows, cols, 1)
-    chunk = max(1, min(n, ws_limit // per, 65535))
+    chunk = _pick_chunk(n, max(1, min(ws_limit // per, 65535)), rows, cols)
     with torch.cuda.device(dev):
         s = _abi.stream_ptr(dev)
         for lo in range(0, n, chunk):

@@ -308,3 +308,14 @@ def test_argument_errors_are_reported_before_any_launch():
     rejected(lib.muon_hip_mfma_probe(tbl, tbl, 2, 10, None, None), EINVAL, "shape")
     rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, (1 << 20) + 1, F32, tbl, None), ESHAPE, "built-in scratch")
     rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, 1, F32, None, None), EINVAL, "null output")
+
+
+def test_chunk_choice_lands_on_whole_rounds():
+    """Matrices per grouped launch: within the workspace cap (plus an eighth), whole rounds of the 256 compute units
+    where the shape allows, never more than the bucket holds, never zero."""
+    pick = muon_utils._pick_chunk
+    assert pick(12288, 248, 768, 2048) == 256  # 6 and 24 tiles per matrix: 6 and 24 whole rounds
+    assert pick(5, 248, 768, 2048) == 5 and pick(1, 7, 4096, 12288) == 1 and pick(100, 1, 4096, 4096) == 1
+    for n, cap, rows, cols in ((72, 15, 4096, 4096), (72, 7, 12288, 4096), (36, 7, 4096, 12288), (24, 91, 896, 4864)):
+        nb = pick(n, cap, rows, cols)
+        assert 1 <= nb <= min(n, cap + cap // 8)
