@@ -204,7 +204,15 @@ int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b,
     return e == hipSuccess ? 0 : hip_fail(e, "sympoly launch");
 }
 
-int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int Kp, int batch, double a, hipStream_t s) {
+// Parameter update folded into the last B.X of a step (parameters with rows <= cols).
+struct FoldUpdate {
+    const void* const* p_ptrs;
+    int p_dtype, rows, cols;
+    double scale, lr, weight_decay;
+};
+
+int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int Kp, int batch, double a, hipStream_t s,
+          const FoldUpdate* fold = nullptr) {
     GemmArgs g = {};
     const int tile = gemm_cfg_tile(cfg);
     g.P = B;
@@ -224,9 +232,18 @@ int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int K
     g.strideEt = blocked_elems(Mp, Kp);
     g.cbEt = Kp / BLK_COLS;
     g.s0 = (float)a;
+    if (fold) {
+        g.upd_ptrs = fold->p_ptrs;
+        g.upd_dtype = fold->p_dtype;
+        g.upd_rows = fold->rows;
+        g.upd_cols = fold->cols;
+        g.upd_scale = (float)fold->scale;
+        g.upd_decay = (float)(1.0 - fold->lr * fold->weight_decay);
+        g.upd_alpha = (float)(-fold->lr);
+    }
     SET_TRACE(g);
     Timed t(MUON_HIP_K_BX, s);
-    hipError_t e = launch_gemm_nt(cfg, EPI_BX, g, s);
+    hipError_t e = launch_gemm_nt(cfg, fold ? EPI_BX_UPD : EPI_BX, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "bx launch");
 }
 
@@ -312,8 +329,12 @@ int muon_hip_normalize(void* workspace, int rows, int cols, int batch, void* str
     return e == hipSuccess ? 0 : hip_fail(e, "normalize launch");
 }
 
-int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int steps, double a, double b, double c,
-                        void* stream) {
+}  // extern "C"
+
+namespace {
+// normalise, then `steps` iterations; with `fold` the last B.X applies the parameter update instead of writing X'
+int ns_chain(void* workspace, int rows, int cols, int batch, int steps, double a, double b, double c, void* stream,
+             const FoldUpdate* fold) {
     Plan p;
     if (int rc = make_plan(rows, cols, batch, p)) return rc;
     if (int rc = check_ws(workspace)) return rc;
@@ -327,10 +348,20 @@ int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int step
     for (int it = 0; it < steps; ++it) {
         if (int rc = do_syrk(pick_cfg(p.M, EPI_SYRK, p.Kp), X[cur], A, p.Mp, p.Kp, batch, s)) return rc;
         if (int rc = do_sympoly(pick_cfg(p.M, EPI_SYMPOLY), A, B, p.Mp, batch, b, c, s)) return rc;
-        if (int rc = do_bx(pick_cfg(p.M, EPI_BX), B, X[cur], X[cur ^ 1], p.Mp, p.Kp, batch, a, s)) return rc;
+        if (int rc = do_bx(pick_cfg(p.M, EPI_BX), B, X[cur], X[cur ^ 1], p.Mp, p.Kp, batch, a, s,
+                           it == steps - 1 ? fold : nullptr))
+            return rc;
         cur ^= 1;
     }
     return 0;
+}
+}  // namespace
+
+extern "C" {
+
+int muon_hip_ns_grouped(void* workspace, int rows, int cols, int batch, int steps, double a, double b, double c,
+                        void* stream) {
+    return ns_chain(workspace, rows, cols, batch, steps, a, b, c, stream, nullptr);
 }
 
 int muon_hip_apply_update(const void* const* p_ptrs, int p_dtype, void* workspace, int rows, int cols, int batch,
@@ -365,6 +396,13 @@ int muon_hip_step_grouped(const void* const* p_ptrs, const void* const* g_ptrs, 
     if (int rc = muon_hip_momentum_norm(g_ptrs, m_ptrs, g_dtype, m_dtype, workspace, rows, cols, batch, beta, nesterov,
                                         write_back_grad, stream))
         return rc;
+    // A parameter that has X's orientation (rows <= cols) is updated by the epilogue of the last B.X: the final
+    // X' is then neither written nor read back.  The others go through the transposing update kernel.
+    if (rows <= cols && ns_steps >= 1) {
+        if (!p_ptrs || !dtype_ok(p_dtype)) return fail(MUON_HIP_EINVAL, "bad pointer table, dtype or steps");
+        const FoldUpdate fold{p_ptrs, p_dtype, rows, cols, scale, lr, weight_decay};
+        return ns_chain(workspace, rows, cols, batch, ns_steps, a, b, c, stream, &fold);
+    }
     if (int rc = muon_hip_ns_grouped(workspace, rows, cols, batch, ns_steps, a, b, c, stream)) return rc;
     return muon_hip_apply_update(p_ptrs, p_dtype, workspace, rows, cols, batch, ns_steps, scale, lr, weight_decay,
                                  stream);

@@ -3,7 +3,9 @@
 #include <hip/hip_runtime.h>
 #include "common.h"
 
-enum { EPI_SYRK = 0, EPI_SYMPOLY = 1, EPI_BX = 2 };
+// EPI_BX_UPD is EPI_BX with the parameter update folded into the epilogue (GemmArgs::upd_*) instead of writing X'
+enum { EPI_SYRK = 0, EPI_SYMPOLY = 1, EPI_BX = 2, EPI_BX_UPD = 3 };
+constexpr bool epi_is_bx(int e) { return e == EPI_BX || e == EPI_BX_UPD; }
 enum {
     GEMM_CFG_128_PIPE = 0,      // 128x128 tile, 4 waves, 64-column k-tiles in two LDS stages
     GEMM_CFG_256_PIPE = 1,      // 256x256 tile, 8 waves, the same pipeline
@@ -30,6 +32,12 @@ struct GemmArgs {
     long strideEt;
     int cbEt;
     float s0, s1;           // SYMPOLY: (b, c); BX: (a, -)
+    // BX, optional: fold apply_scaling and the parameter update into the epilogue instead of writing X'
+    // (parameters in the orientation of X only, i.e. rows <= cols)
+    const void* const* upd_ptrs;  // device table of parameter base pointers, one per matrix; null = write X'
+    int upd_dtype;                // MUON_HIP_F32 or MUON_HIP_BF16
+    int upd_rows, upd_cols;       // the parameter's own (unpadded) shape
+    float upd_scale, upd_decay, upd_alpha;  // python-double scale, 1 - lr*wd and -lr, as fp32
     int big_blocks;         // set by the launcher: workgroups that compute whole 256x256 tiles (split-tail kernel)
 #ifdef MUON_TILE_TRACE
     long* trace;            // measurement builds only: 8 longs per workgroup

@@ -81,7 +81,7 @@ __device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int logical) {
     const int bidx = logical / g.tiles_per_mat;
     const int t = logical - bidx * g.tiles_per_mat;
     int ti = 0, tj = 0;  // plain locals: references into the struct kept it in scratch memory
-    if (EPI == EPI_BX) rect_decode<4>(t, g.tiles_m, g.tiles_n, ti, tj);
+    if (epi_is_bx(EPI)) rect_decode<4>(t, g.tiles_m, g.tiles_n, ti, tj);
     else tri_decode<4>(t, g.tiles_m, ti, tj);
     return TileCoord{bidx, ti, tj};
 }
@@ -159,7 +159,7 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN, quad = lane >> 4;
     const int m0 = tc.ti * BM, n0 = tc.tj * BN;
-    const bool diag = (EPI != EPI_BX) && (tc.ti == tc.tj);
+    const bool diag = (!epi_is_bx(EPI)) && (tc.ti == tc.tj);
     // Et and Ct hold the tile as rows n0.. (BN of them) x columns m0.. (BM of them).  Chunk c of a
     // thread: 16 bytes j = c%8 of the 128-byte row piece of row n = (c/8)%BN in column block c/8/BN,
     // so that a wave touches 8 rows x 128 bytes = 1 KB of one block, contiguous in memory.
@@ -257,7 +257,53 @@ __device__ __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc,
 template <int BM, int BN>
 constexpr int epilogue_nn_bytes() { return BM * (BN * 2 + 16); }
 
-template <int BM, int BN, int WGM, int WGN>
+// Folded parameter update: eight consecutive elements of one parameter row, o = bf16(X' * scale);
+// p <- rnd(p * decay); p <- rnd(p + alpha * o), the arithmetic of the stand-alone update kernel (elementwise.hip).
+// The parameter piece is fetched into registers early (fold_load) and applied after the tile has been through LDS.
+struct FoldPiece {
+    f32x4 lo;  // bf16 parameter: the eight values; fp32 parameter: the first four (the other four are fetched
+               // when the piece is applied, from the cache line that this fetch brought in)
+};
+template <typename PT>
+__device__ __forceinline__ FoldPiece fold_load(const PT* p, bool vec, int left) {
+    FoldPiece f;
+    f.lo = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (vec && left >= 8) f.lo = __builtin_nontemporal_load((const f32x4*)p);
+    return f;
+}
+template <typename PT>
+__device__ __forceinline__ void fold_apply(PT* p, const FoldPiece& f, const bf16x8& x, bool vec, int left, const GemmArgs& g) {
+    constexpr bool PBF = std::is_same<PT, bf16_t>::value;
+    auto one = [&](float pv, bf16_t xv) {
+        const float os = rbf(bf2f(xv) * g.upd_scale);
+        const float pd = PBF ? rbf(pv * g.upd_decay) : pv * g.upd_decay;
+        return fmaf(g.upd_alpha, os, pd);
+    };
+    if (vec && left >= 8) {
+        if constexpr (PBF) {
+            bf16x8 pv = *(const bf16x8*)&f.lo;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) pv[k] = f2bf(one(bf2f(pv[k]), x[k]));
+            __builtin_nontemporal_store(pv, (bf16x8*)p);
+        } else {
+            f32x4 a = f.lo, b = __builtin_nontemporal_load((const f32x4*)(p + 4));
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                a[k] = one(a[k], x[k]);
+                b[k] = one(b[k], x[4 + k]);
+            }
+            __builtin_nontemporal_store(a, (f32x4*)p);
+            __builtin_nontemporal_store(b, (f32x4*)(p + 4));
+        }
+    } else {  // ragged row end or unaligned parameter: element by element
+        for (int k = 0; k < 8 && k < left; ++k) {
+            if constexpr (PBF) p[k] = f2bf(one(bf2f(p[k]), x[k]));
+            else p[k] = one(p[k], x[k]);
+        }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN, bool FOLD>
 __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& tc,
                                             f32x4 (&acc)[BM / WGM / 16][BN / WGN / 16], unsigned char* smem) {
     constexpr int NT = WGM * WGN * 64;
@@ -270,10 +316,27 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN, quad = lane >> 4;
     const int m0 = tc.ti * BM, n0 = tc.tj * BN;
-    // chunk c: 16 bytes j of the row piece of row m in column block cbk of the tile; a wave covers 16 rows of
-    // one block = 1 KB contiguous in memory
+    // Last iteration of a step, parameter in the orientation of X: the scaled update goes straight into the
+    // parameter (apply_scaling and the decay / update lines, muon_utils.py:167-175, :324-325) and X' is not written.
+    constexpr bool fold = FOLD;
+    // chunk c: 16 bytes j of the row piece of row m in column block cbk of the tile.  Writing X' a wave covers
+    // 16 rows of one block = 1 KB contiguous in the blocked layout; writing the parameter (row-major) it covers
+    // whole tile rows instead, 2 x 512 B of bf16, and reads E in 64-byte pieces.
+    auto decode = [&](int c, int& j, int& m, int& cbk) {
+        if constexpr (fold) {
+            const int piece = c % (BN / 8);
+            m = c / (BN / 8);
+            cbk = piece / CPB;
+            j = piece % CPB;
+        } else {
+            j = c % CPB;
+            m = (c / CPB) % BM;
+            cbk = (c / CPB) / BM;
+        }
+    };
     auto tile_chunk = [&](int c, int cb, long& goff, int& loff) {
-        const int j = c % CPB, m = (c / CPB) % BM, cbk = (c / CPB) / BM;
+        int j, m, cbk;
+        decode(c, j, m, cbk);
         goff = panel_offset(m0, cb) + (long)((n0 >> BLK_SHIFT) + cbk) * BLK_ELEMS + m * BLK_COLS + j * 8;
         loff = m * S + (cbk * CPB + j) * 16;
     };
@@ -296,18 +359,58 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
             for (int r = 0; r < 4; ++r) t[r] = f2bf(acc[i][j][r]);
             *(bf16x4*)(smem + (wm * WTM + i * 16 + (lane & 15)) * S + (wn * WTN + j * 16 + quad * 4) * 2) = t;
         }
-    __syncthreads();
     bf16_t* C = g.C + tc.bidx * g.strideC;
+    if constexpr (!fold) {
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < NLE; ++u) {
+            long goff;
+            int loff;
+            tile_chunk(tid + u * NT, g.cbC, goff, loff);
+            const bf16x8 t = *(const bf16x8*)(smem + loff);
+            bf16x8 o;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) o[k] = f2bf(rbf(g.s0 * bf2f(ev[u][k])) + bf2f(t[k]));
+            *(bf16x8*)(C + goff) = o;
+        }
+        return;
+    }
+    void* pbase = const_cast<void*>(g.upd_ptrs[tc.bidx]);
+    const bool pvec = (g.upd_cols % 8 == 0) && ((((uintptr_t)pbase) & 15) == 0);
+    const bool pbf = g.upd_dtype == MUON_HIP_BF16;
+    // The parameter pieces are fetched here, with the accumulators already in LDS, so that their latency passes
+    // behind the barrier.
+    auto piece = [&](int c, long& poff, int& left) {
+        int j, m, cbk;
+        decode(c, j, m, cbk);
+        const int row = m0 + m, col = n0 + cbk * BLK_COLS + j * 8;
+        poff = (long)row * g.upd_cols + col;
+        left = g.upd_cols - col;
+        return row < g.upd_rows && left > 0;
+    };
+    FoldPiece pv[NLE];
 #pragma unroll
     for (int u = 0; u < NLE; ++u) {
-        long goff;
-        int loff;
-        tile_chunk(tid + u * NT, g.cbC, goff, loff);
+        long poff;
+        int left;
+        if (piece(tid + u * NT, poff, left))
+            pv[u] = pbf ? fold_load<bf16_t>((const bf16_t*)pbase + poff, pvec, left) : fold_load<float>((const float*)pbase + poff, pvec, left);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int u = 0; u < NLE; ++u) {
+        long goff, poff;
+        int loff, left;
+        const int c = tid + u * NT;
+        tile_chunk(c, g.cbC, goff, loff);
         const bf16x8 t = *(const bf16x8*)(smem + loff);
         bf16x8 o;
 #pragma unroll
         for (int k = 0; k < 8; ++k) o[k] = f2bf(rbf(g.s0 * bf2f(ev[u][k])) + bf2f(t[k]));
-        *(bf16x8*)(C + goff) = o;
+        if (piece(c, poff, left)) {
+            if (pbf) fold_apply<bf16_t>((bf16_t*)pbase + poff, pv[u], o, pvec, left, g);
+            else fold_apply<float>((float*)pbase + poff, pv[u], o, pvec, left, g);
+        }
     }
 }
 
@@ -361,7 +464,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     constexpr int KS = 2;  // 32-column MFMA steps per k-tile
     constexpr int NMF = FM * FN, NRD = FM + FN, NLD = LA + LB;
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "dma split");
-    static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
+    static_assert(epi_is_bx(EPI) || BM == BN, "triangular tiles are square");
 
     extern __shared__ __align__(16) unsigned char smem[];
 
@@ -369,7 +472,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const TileCoord tc = decode_tile<EPI>(g);
-    constexpr bool QT = EPI == EPI_BX;  // Q is X itself, rows = reduction index
+    constexpr bool QT = epi_is_bx(EPI);  // Q is X itself, rows = reduction index
     const int kb = g.kdim / BLK_COLS;
     const bf16_t* Pb = g.P + tc.bidx * g.strideP + panel_offset(tc.ti * BM, kb);
     const bf16_t* Qb = g.Q + tc.bidx * g.strideQ +
@@ -492,7 +595,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
         }
     }
     WAIT_VM(0);  // the dummy loads of the last two tails must not land in the epilogue's tile
-    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN>(g, tc, acc, smem);
+    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN, EPI == EPI_BX_UPD>(g, tc, acc, smem);
     else epilogue<BM, BN, WGM, WGN, EPI, false>(g, tc, acc, smem);
 }
 
@@ -545,13 +648,13 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     static_assert(FM * FN <= 32, "one mask bit per fragment");
     static_assert(NW == 8, "two groups of four waves, one of each per SIMD");
     static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "dma split");
-    static_assert(EPI == EPI_BX || BM == BN, "triangular tiles are square");
+    static_assert(epi_is_bx(EPI) || BM == BN, "triangular tiles are square");
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int grp = wave >> 2;
     const int wm = wave / WGN, wn = wave % WGN;
-    constexpr bool QT = EPI == EPI_BX;  // Q is X itself, rows = reduction index
+    constexpr bool QT = epi_is_bx(EPI);  // Q is X itself, rows = reduction index
     const int kb = g.kdim / BLK_COLS;
     const bf16_t* Pb = uniform_ptr(g.P + tc.bidx * g.strideP + panel_offset(tc.ti * BM, kb));
     const bf16_t* Qb = uniform_ptr(g.Q + tc.bidx * g.strideQ +
@@ -611,7 +714,7 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     // Diagonal tile of a symmetric product: a fragment of a wave that lies entirely below the diagonal is the
     // mirror image of one another wave computes, and the epilogue does not read it.  Bit i*FN+j of a wave's mask:
     // skip that fragment's MFMAs (and the fragment reads nobody needs).
-    const bool diag = EPI != EPI_BX && tc.ti == tc.tj;
+    const bool diag = !epi_is_bx(EPI) && tc.ti == tc.tj;
     // fragment reads: lane l takes row l%16 of the fragment and the 16-byte chunk l/16 of its 64-byte row
     // (chunk c of row r sits at c ^ pp_swizzle((r>>2)&3))
     const int sw = pp_swizzle((lane >> 2) & 3), kq = lane >> 4;
@@ -721,7 +824,7 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     if (!grp) __builtin_amdgcn_s_barrier();
     MUON_TRACE_STAMP(g, 2);
     WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
-    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN>(g, tc, acc, smem);
+    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN, EPI == EPI_BX_UPD>(g, tc, acc, smem);
     else epilogue<BM, BN, WGM, WGN, EPI, true>(g, tc, acc, smem);
 }
 
@@ -746,7 +849,7 @@ __global__ void __launch_bounds__(512) gemm_nt_pp_tail_kernel(const GemmArgs g) 
     } else {
         const int s = blockIdx.x - g.big_blocks, quarter = s & 3;
         TileCoord tc = tile_of<EPI>(g, g.big_blocks + (s >> 2));
-        if (EPI != EPI_BX && tc.ti == tc.tj && quarter == 2) return;
+        if (!epi_is_bx(EPI) && tc.ti == tc.tj && quarter == 2) return;
         tc.ti = tc.ti * 2 + (quarter >> 1);
         tc.tj = tc.tj * 2 + (quarter & 1);
         pp_tile<128, 128, 2, 4, EPI>(g, tc, smem);
@@ -756,7 +859,7 @@ __global__ void __launch_bounds__(512) gemm_nt_pp_tail_kernel(const GemmArgs g) 
 template <int BM, int BN, int WGM, int WGN, int EPI, int FEED>
 hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
     constexpr int stages = 2 * (BM + BN) * ROW_BYTES;
-    constexpr int epi = EPI == EPI_BX ? epilogue_nn_bytes<BM, BN>() : epilogue_bytes<BM, BN>();
+    constexpr int epi = epi_is_bx(EPI) ? epilogue_nn_bytes<BM, BN>() : epilogue_bytes<BM, BN>();
     constexpr int smem = stages > epi ? stages : epi;
     static std::atomic<bool> configured{false};  // per instantiation; setting the attribute twice is harmless
     void (*kern)(const GemmArgs);
@@ -795,7 +898,7 @@ int gemm_cfg_tile(int cfg) {
 template <int EPI>
 hipError_t launch_pp_tail(GemmArgs g, int nblocks, int rest, hipStream_t stream) {
     constexpr int stages = 2 * (256 + 256) * ROW_BYTES;
-    constexpr int epi = EPI == EPI_BX ? epilogue_nn_bytes<256, 256>() : epilogue_bytes<256, 256>();
+    constexpr int epi = epi_is_bx(EPI) ? epilogue_nn_bytes<256, 256>() : epilogue_bytes<256, 256>();
     constexpr int smem = stages > epi ? stages : epi;  // the 128-tiles need less of both
     static std::atomic<bool> configured{false};
     auto kern = gemm_nt_pp_tail_kernel<EPI>;
@@ -820,6 +923,7 @@ hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t strea
             case EPI_SYRK: return launch_pp_tail<EPI_SYRK>(g, nblocks, rest, stream);
             case EPI_SYMPOLY: return launch_pp_tail<EPI_SYMPOLY>(g, nblocks, rest, stream);
             case EPI_BX: return launch_pp_tail<EPI_BX>(g, nblocks, rest, stream);
+            case EPI_BX_UPD: return launch_pp_tail<EPI_BX_UPD>(g, nblocks, rest, stream);
             default: return hipErrorInvalidValue;
         }
     }
@@ -827,6 +931,7 @@ hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t strea
         case EPI_SYRK: return launch_cfg<EPI_SYRK>(cfg, g, nblocks, stream);
         case EPI_SYMPOLY: return launch_cfg<EPI_SYMPOLY>(cfg, g, nblocks, stream);
         case EPI_BX: return launch_cfg<EPI_BX>(cfg, g, nblocks, stream);
+        case EPI_BX_UPD: return launch_cfg<EPI_BX_UPD>(cfg, g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }

@@ -477,6 +477,45 @@ def test_grouped_equals_per_matrix_bitwise(env):
         assert torch.equal(p.detach(), q.detach())
 
 
+@pytest.mark.parametrize("pdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols,batch", [(256, 384, 3), (37, 53, 2), (100, 300, 2), (512, 1024, 2), (768, 2048, 3), (64, 64, 1)])
+def test_folded_update_equals_the_staged_sequence_bitwise(env, pdtype, rows, cols, batch):
+    """muon_hip_step_grouped lets the epilogue of the last B.X apply the scaled update to a parameter that has X's
+    orientation (rows <= cols), without writing the final X'.  The stage entry points run the same arithmetic through
+    the stand-alone update kernel (itself bit-identical to torch on the device): parameters and momentum must come out
+    equal bit for bit, ragged shapes and both parameter dtypes included."""
+    print(f"folded update {pdtype} {rows}x{cols} x{batch}", flush=True)
+    lib, abi, mu, dev = env["lib"], env["abi"], env["mu"], env["dev"]
+    gen = torch.Generator().manual_seed(rows * 13 + cols)
+    gdt = torch.bfloat16 if pdtype == torch.bfloat16 else torch.float32
+    p0 = [(0.02 * torch.randn(rows, cols, generator=gen)).to(pdtype).to(dev) for _ in range(batch)]
+    g0 = [(1e-3 * torch.randn(rows, cols, generator=gen)).to(gdt).to(dev) for _ in range(batch)]
+    m0 = [(1e-3 * torch.randn(rows, cols, generator=gen)).to(dev) for _ in range(batch)]
+    a, b, c = env["O"].NS_COEFFS
+    lr, wd, beta, steps = 0.02, 0.01, 0.95, 5
+    scale = mu.scale_factor(rows, cols, True)
+    outs = []
+    for fused in (True, False):
+        p, g, m = [t.clone() for t in p0], [t.clone() for t in g0], [t.clone() for t in m0]
+        ws = torch.empty(abi.workspace_bytes(rows, cols, batch), dtype=torch.uint8, device=dev)
+        table = torch.tensor([t.data_ptr() for t in p + g + m], dtype=torch.int64, device=dev)
+        tp, tg, tm = table.data_ptr(), table.data_ptr() + 8 * batch, table.data_ptr() + 16 * batch
+        codes = (abi.dtype_code(pdtype), abi.dtype_code(gdt), abi.F32)
+        if fused:
+            abi.check(lib.muon_hip_step_grouped(tp, tg, tm, *codes, ws.data_ptr(), rows, cols, batch, lr, wd, beta, 1, steps,
+                                                scale, a, b, c, 0, 0))
+        else:
+            abi.check(lib.muon_hip_momentum_norm(tg, tm, codes[1], codes[2], ws.data_ptr(), rows, cols, batch, beta, 1, 0, 0))
+            abi.check(lib.muon_hip_ns_grouped(ws.data_ptr(), rows, cols, batch, steps, a, b, c, 0))
+            abi.check(lib.muon_hip_apply_update(tp, codes[0], ws.data_ptr(), rows, cols, batch, steps, scale, lr, wd, 0))
+        torch.cuda.synchronize()
+        outs.append((p, m))
+    for i in range(batch):
+        assert torch.equal(outs[0][1][i], outs[1][1][i])
+        assert torch.equal(outs[0][0][i], outs[1][0][i]), f"matrix {i}: {(outs[0][0][i] != outs[1][0][i]).sum().item()} elements differ"
+        assert not torch.equal(outs[0][0][i], p0[i]), "the parameter moved"
+
+
 def test_grouped_equals_per_matrix_bitwise_on_256_tiles(env):
     """The same for shapes whose short side is a whole number of 256-tiles (ping-pong and split-tail kernels) and
     for the expert shapes 768x2048 / 2048x768 (128-tiles): bf16 parameters, fp32 momentum, three matrices per
