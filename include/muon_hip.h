@@ -56,7 +56,8 @@ extern "C" {
 #define MUON_HIP_CFG_128_PIPE 0      /* 128x128 tile, 4 waves, 64-column k-tiles, two LDS stages */
 #define MUON_HIP_CFG_256_PIPE 1      /* 256x256 tile, 8 waves, the same pipeline */
 #define MUON_HIP_CFG_256_PINGPONG 2  /* 256x256 tile, two groups of 4 waves alternating memory / MFMA phases */
-#define MUON_HIP_CFG_COUNT 3
+#define MUON_HIP_CFG_128_PINGPONG 3  /* 128x128 tile, the same eight-wave kernel, two workgroups per compute unit */
+#define MUON_HIP_CFG_COUNT 4
 
 int muon_hip_version(void);
 const char* muon_hip_last_error(void);

@@ -87,14 +87,15 @@ inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
 // Tile edge for a matrix whose short side is M: 256 when M is a whole number of 256-tiles.
 bool use_tile256(int M) { return M % 256 == 0 && M >= 512; }
 
-// Configuration per kernel, from a sweep of every variant over the benchmark shapes: the ping-pong
-// kernel wherever 256-tiles fill the machine, 128-tiles for the symmetric products of small matrices.
+// Configuration per kernel, from a sweep of every variant over the benchmark shapes: the ping-pong kernel
+// everywhere, on 256-tiles where they fill the machine and on 128-tiles (two workgroups per compute unit) for
+// short sides that are no whole number of 256-tiles and for the symmetric products of matrices up to 512 rows.
 int pick_cfg(int M, int epi = EPI_BX, int kdim = 0) {
     const int forced = g_forced_cfg.load(std::memory_order_relaxed);
     if (forced != MUON_HIP_CFG_AUTO) return forced;
     (void)kdim;
-    if (!use_tile256(M)) return GEMM_CFG_128_PIPE;
-    if (epi != EPI_BX && M <= 512) return GEMM_CFG_128_PIPE;
+    if (!use_tile256(M)) return GEMM_CFG_128_PINGPONG;
+    if (epi != EPI_BX && M <= 512) return GEMM_CFG_128_PINGPONG;
     return GEMM_CFG_256_PINGPONG;
 }
 

@@ -10,7 +10,8 @@ enum {
     GEMM_CFG_128_PIPE = 0,      // 128x128 tile, 4 waves, 64-column k-tiles in two LDS stages
     GEMM_CFG_256_PIPE = 1,      // 256x256 tile, 8 waves, the same pipeline
     GEMM_CFG_256_PINGPONG = 2,  // 256x256 tile, 8 waves in two alternating groups, four stages of 32 columns
-    GEMM_CFG_COUNT = 3
+    GEMM_CFG_128_PINGPONG = 3,  // 128x128 tile, the same eight-wave kernel, two workgroups per compute unit
+    GEMM_CFG_COUNT = 4
 };
 
 struct GemmArgs {

@@ -880,6 +880,7 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
         case GEMM_CFG_128_PIPE: return launch_one<128, 128, 2, 2, EPI, 0>(g, nblocks, stream);
         case GEMM_CFG_256_PIPE: return launch_one<256, 256, 2, 4, EPI, 0>(g, nblocks, stream);
         case GEMM_CFG_256_PINGPONG: return launch_one<256, 256, 2, 4, EPI, 1>(g, nblocks, stream);
+        case GEMM_CFG_128_PINGPONG: return launch_one<128, 128, 2, 4, EPI, 1>(g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -888,7 +889,8 @@ hipError_t launch_cfg(int cfg, const GemmArgs& g, int nblocks, hipStream_t strea
 
 int gemm_cfg_tile(int cfg) {
     switch (cfg) {
-        case GEMM_CFG_128_PIPE: return 128;
+        case GEMM_CFG_128_PIPE:
+        case GEMM_CFG_128_PINGPONG: return 128;
         case GEMM_CFG_256_PIPE:
         case GEMM_CFG_256_PINGPONG: return 256;
         default: return 0;

@@ -104,7 +104,7 @@ def matmul_transpose_assign(d_in: Tensor, d_out: Tensor) -> None:
         raise TypeError(f"the MI355X kernel multiplies bfloat16 operands, got {d_in.dtype}")
     M, K = d_in.shape
     tile = 256 if (M % 256 == 0 and M >= 512) else 128
-    cfg = _abi.CFG_AUTO if tile == 256 else _abi.CFG_128_PIPE
+    cfg = _abi.CFG_AUTO  # the library picks the kernel for the padded size
     Mp, Kp = -(-M // tile) * tile, -(-K // tile) * tile
     lib = _abi.lib()
     with torch.cuda.device(d_in.device):
@@ -127,6 +127,7 @@ def get_autotune_config():
         dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=64, num_stages=2, num_warps=4, config=_abi.CFG_128_PIPE),
         dict(BLOCK_SIZE_M=256, BLOCK_SIZE_N=256, BLOCK_SIZE_K=64, num_stages=2, num_warps=8, config=_abi.CFG_256_PIPE),
         dict(BLOCK_SIZE_M=256, BLOCK_SIZE_N=256, BLOCK_SIZE_K=32, num_stages=4, num_warps=8, config=_abi.CFG_256_PINGPONG),
+        dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=32, num_stages=4, num_warps=8, config=_abi.CFG_128_PINGPONG),
     ]
 
 

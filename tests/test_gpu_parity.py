@@ -47,7 +47,7 @@ def _assert_product_close(got, ref64, absprod):
     assert not bad.any(), f"{int(bad.sum())} elements outside one bf16 ulp"
 
 
-CFGS = list(range(3))
+CFGS = list(range(4))
 
 
 def _pack(env, t):
