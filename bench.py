@@ -426,9 +426,12 @@ def main():
     bx_f = 2.0 * syrk_f
     gb = 2 if pd == torch.bfloat16 else 4
     mom_bytes = elements * (gb + 2 * 4 + 2) if md == torch.float32 or pd == torch.float32 else elements * (3 * gb + 2)
+    # The update kernel runs only for parameters with rows > cols (X is their transpose); the others are updated by
+    # the epilogue of the last B.X of the step, whose time is inside bx_axpy.
+    upd_elements = sum(s[0] * s[1] for s in shapes if s[0] > s[1]) if HP["ns_steps"] >= 1 else elements
     work = {"syrk": (syrk_f, "flop"), "sympoly": (symp_f, "flop"), "bx_axpy": (bx_f, "flop"),
             "momentum_norm": (mom_bytes, "byte"), "normalize": (elements * 4, "byte"),
-            "apply_update": (elements * (2 + 2 * gb), "byte")}
+            "apply_update": (upd_elements * (2 + 2 * gb), "byte")}
     kernels = {}
     for name, (tot_ms, cnt) in kern.items():
         if cnt == 0 or name not in work:
@@ -447,7 +450,9 @@ def main():
     if "bx_axpy" in kernels:
         tot_ms, cnt = kern["bx_axpy"]
         achieved = bx_f * args.steps / (tot_ms * 1e-3) / 1e12
-        roofline = {"kernel": "gemm_nt_pp_kernel<256, 256, 2, 4, EPI_BX> (X' = a.X + B.X)", "bound": "mfma", "achieved": achieved,
+        roofline = {"kernel": "gemm_nt_pp_kernel<256, 256, 2, 4, EPI_BX> (X' = a.X + B.X; the last of a step's five launches per "
+                              "chunk is EPI_BX_UPD, the same product with the parameter update in its epilogue)",
+                    "bound": "mfma", "achieved": achieved,
                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                     "traffic": recorded_traffic(args.workload) if layers == w["layers"] else None,
                     "launches": cnt, "avg_launch_ms": tot_ms / cnt,
