@@ -426,9 +426,9 @@ def main():
     bx_f = 2.0 * syrk_f
     gb = 2 if pd == torch.bfloat16 else 4
     mom_bytes = elements * (gb + 2 * 4 + 2) if md == torch.float32 or pd == torch.float32 else elements * (3 * gb + 2)
-    # The update kernel runs only for parameters with rows > cols (X is their transpose); the others are updated by
-    # the epilogue of the last B.X of the step, whose time is inside bx_axpy.
-    upd_elements = sum(s[0] * s[1] for s in shapes if s[0] > s[1]) if HP["ns_steps"] >= 1 else elements
+    # With at least one iteration the parameters are updated by the epilogue of the last B.X of the step (its time is
+    # inside bx_axpy) and the update kernel does not run: it appears below only if it was launched.
+    upd_elements = elements
     work = {"syrk": (syrk_f, "flop"), "sympoly": (symp_f, "flop"), "bx_axpy": (bx_f, "flop"),
             "momentum_norm": (mom_bytes, "byte"), "normalize": (elements * 4, "byte"),
             "apply_update": (upd_elements * (2 + 2 * gb), "byte")}

@@ -114,7 +114,10 @@ int muon_hip_apply_update(const void* const* p_ptrs, int p_dtype, void* workspac
 int muon_hip_ns_output(void* workspace, int rows, int cols, int batch, int steps, void* out, void* stream);
 
 /* The whole Muon step for one bucket: SingelDeviceWork.start (muon_utils.py:315-325) for
- * `batch` same-shape parameters in one grouped dispatch per stage. */
+ * `batch` same-shape parameters in one grouped dispatch per stage.  With ns_steps >= 1 the scaling,
+ * decay and update lines (:167-175, :324-325) run in the epilogue of the last B.X product, so the
+ * final X' is neither written nor read back (results equal muon_hip_momentum_norm + muon_hip_ns_grouped
+ * + muon_hip_apply_update bit for bit); the workspace then does not hold the last iterate. */
 int muon_hip_step_grouped(const void* const* p_ptrs, const void* const* g_ptrs, const void* const* m_ptrs,
                           int p_dtype, int g_dtype, int m_dtype, void* workspace, int rows, int cols, int batch,
                           double lr, double weight_decay, double beta, int nesterov, int ns_steps, double scale,

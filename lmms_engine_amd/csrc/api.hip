@@ -205,7 +205,7 @@ int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b,
     return e == hipSuccess ? 0 : hip_fail(e, "sympoly launch");
 }
 
-// Parameter update folded into the last B.X of a step (parameters with rows <= cols).
+// Parameter update folded into the last B.X of a step (the parameter is X's image when rows <= cols, its transpose otherwise).
 struct FoldUpdate {
     const void* const* p_ptrs;
     int p_dtype, rows, cols;
@@ -244,7 +244,7 @@ int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int K
     }
     SET_TRACE(g);
     Timed t(MUON_HIP_K_BX, s);
-    hipError_t e = launch_gemm_nt(cfg, fold ? EPI_BX_UPD : EPI_BX, g, s);
+    hipError_t e = launch_gemm_nt(cfg, !fold ? EPI_BX : fold->rows <= fold->cols ? EPI_BX_UPD : EPI_BX_UPD_T, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "bx launch");
 }
 
@@ -397,9 +397,9 @@ int muon_hip_step_grouped(const void* const* p_ptrs, const void* const* g_ptrs, 
     if (int rc = muon_hip_momentum_norm(g_ptrs, m_ptrs, g_dtype, m_dtype, workspace, rows, cols, batch, beta, nesterov,
                                         write_back_grad, stream))
         return rc;
-    // A parameter that has X's orientation (rows <= cols) is updated by the epilogue of the last B.X: the final
-    // X' is then neither written nor read back.  The others go through the transposing update kernel.
-    if (rows <= cols && ns_steps >= 1) {
+    // The parameter is updated by the epilogue of the last B.X (for rows > cols through a transposing gather out of
+    // LDS): the final X' is then neither written nor read back.  Without an iteration there is no such product.
+    if (ns_steps >= 1) {
         if (!p_ptrs || !dtype_ok(p_dtype)) return fail(MUON_HIP_EINVAL, "bad pointer table, dtype or steps");
         const FoldUpdate fold{p_ptrs, p_dtype, rows, cols, scale, lr, weight_decay};
         return ns_chain(workspace, rows, cols, batch, ns_steps, a, b, c, stream, &fold);

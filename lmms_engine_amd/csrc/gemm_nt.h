@@ -3,9 +3,12 @@
 #include <hip/hip_runtime.h>
 #include "common.h"
 
-// EPI_BX_UPD is EPI_BX with the parameter update folded into the epilogue (GemmArgs::upd_*) instead of writing X'
-enum { EPI_SYRK = 0, EPI_SYMPOLY = 1, EPI_BX = 2, EPI_BX_UPD = 3 };
-constexpr bool epi_is_bx(int e) { return e == EPI_BX || e == EPI_BX_UPD; }
+// EPI_BX_UPD is EPI_BX with the parameter update folded into the epilogue (GemmArgs::upd_*) instead of writing X';
+// EPI_BX_UPD_T is the same for a parameter that is the transpose of X (rows > cols)
+enum { EPI_SYRK = 0, EPI_SYMPOLY = 1, EPI_BX = 2, EPI_BX_UPD = 3, EPI_BX_UPD_T = 4 };
+constexpr bool epi_is_bx(int e) { return e == EPI_BX || e == EPI_BX_UPD || e == EPI_BX_UPD_T; }
+// how the B.X epilogue finishes: 0 writes X', 1 updates a parameter in the orientation of X, 2 a transposed one
+constexpr int epi_fold_mode(int e) { return e == EPI_BX_UPD ? 1 : e == EPI_BX_UPD_T ? 2 : 0; }
 enum {
     GEMM_CFG_128_PIPE = 0,      // 128x128 tile, 4 waves, 64-column k-tiles in two LDS stages
     GEMM_CFG_256_PIPE = 1,      // 256x256 tile, 8 waves, the same pipeline
@@ -34,7 +37,7 @@ struct GemmArgs {
     int cbEt;
     float s0, s1;           // SYMPOLY: (b, c); BX: (a, -)
     // BX, optional: fold apply_scaling and the parameter update into the epilogue instead of writing X'
-    // (parameters in the orientation of X only, i.e. rows <= cols)
+    // (EPI_BX_UPD: the parameter is X's image, rows <= cols; EPI_BX_UPD_T: its transpose, rows > cols)
     const void* const* upd_ptrs;  // device table of parameter base pointers, one per matrix; null = write X'
     int upd_dtype;                // MUON_HIP_F32 or MUON_HIP_BF16
     int upd_rows, upd_cols;       // the parameter's own (unpadded) shape

@@ -303,7 +303,7 @@ __device__ __forceinline__ void fold_apply(PT* p, const FoldPiece& f, const bf16
     }
 }
 
-template <int BM, int BN, int WGM, int WGN, bool FOLD>
+template <int BM, int BN, int WGM, int WGN, int FOLD>
 __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& tc,
                                             f32x4 (&acc)[BM / WGM / 16][BN / WGN / 16], unsigned char* smem) {
     constexpr int NT = WGM * WGN * 64;
@@ -318,7 +318,7 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
     const int m0 = tc.ti * BM, n0 = tc.tj * BN;
     // Last iteration of a step, parameter in the orientation of X: the scaled update goes straight into the
     // parameter (apply_scaling and the decay / update lines, muon_utils.py:167-175, :324-325) and X' is not written.
-    constexpr bool fold = FOLD;
+    constexpr bool fold = FOLD == 1;
     // chunk c: 16 bytes j of the row piece of row m in column block cbk of the tile.  Writing X' a wave covers
     // 16 rows of one block = 1 KB contiguous in the blocked layout; writing the parameter (row-major) it covers
     // whole tile rows instead, 2 x 512 B of bf16, and reads E in 64-byte pieces.
@@ -360,7 +360,7 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
             *(bf16x4*)(smem + (wm * WTM + i * 16 + (lane & 15)) * S + (wn * WTN + j * 16 + quad * 4) * 2) = t;
         }
     bf16_t* C = g.C + tc.bidx * g.strideC;
-    if constexpr (!fold) {
+    if constexpr (FOLD == 0) {
         __syncthreads();
 #pragma unroll
         for (int u = 0; u < NLE; ++u) {
@@ -372,6 +372,65 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
 #pragma unroll
             for (int k = 0; k < 8; ++k) o[k] = f2bf(rbf(g.s0 * bf2f(ev[u][k])) + bf2f(t[k]));
             *(bf16x8*)(C + goff) = o;
+        }
+        return;
+    }
+    if constexpr (FOLD == 2) {
+        // The parameter is the transpose of X (rows > cols): row n0 + n of the parameter is column n of the tile.  The
+        // finished X' values go back into T in place, and after a barrier a wave gathers them the other way round with
+        // ds_read_b64_tr_b16 (the gather of the symmetric epilogue): lane i16 of a group of 16 receives
+        // T[m .. m+7][4c + i16 % 4] with m = strip * 128 + grp * 32 + (i16 / 4) * 8, i.e. 16 bytes of row 4c + i16 % 4
+        // of the parameter tile; a wave instruction covers 4 parameter rows x 128 columns.
+        constexpr int NSTRIP = BM / 128, NQUAD = BN / 4, NWV = NT / 64;
+        constexpr int NUNIT = NSTRIP * NQUAD / NWV;
+        static_assert(BM % 128 == 0 && (NSTRIP * NQUAD) % NWV == 0, "whole 128-row strips per wave");
+        void* pbase = const_cast<void*>(g.upd_ptrs[tc.bidx]);
+        const bool pvec = (g.upd_cols % 8 == 0) && ((((uintptr_t)pbase) & 15) == 0);
+        const bool pbf = g.upd_dtype == MUON_HIP_BF16;
+        const int grp = lane >> 4, i16 = lane & 15;
+        auto piece = [&](int u, long& poff, int& left) {
+            const int wu = wave + u * NWV, strip = wu % NSTRIP, c = wu / NSTRIP;
+            const int row = n0 + c * 4 + (i16 & 3), col = m0 + strip * 128 + grp * 32 + (i16 >> 2) * 8;
+            poff = (long)row * g.upd_cols + col;
+            left = g.upd_cols - col;
+            return row < g.upd_rows && left > 0;
+        };
+        FoldPiece pv[NUNIT];
+#pragma unroll
+        for (int u = 0; u < NUNIT; ++u) {
+            long poff;
+            int left;
+            if (piece(u, poff, left))
+                pv[u] = pbf ? fold_load<bf16_t>((const bf16_t*)pbase + poff, pvec, left) : fold_load<float>((const float*)pbase + poff, pvec, left);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < NLE; ++u) {
+            long goff;
+            int loff;
+            tile_chunk(tid + u * NT, g.cbC, goff, loff);
+            const bf16x8 t = *(const bf16x8*)(smem + loff);
+            bf16x8 o;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) o[k] = f2bf(rbf(g.s0 * bf2f(ev[u][k])) + bf2f(t[k]));
+            *(bf16x8*)(smem + loff) = o;
+        }
+        __syncthreads();
+        // lane j = 4r+s of a group addresses row m + 8s + r of T (then + 4), columns 4c..4c+3
+        const unsigned char* src = smem + ((i16 & 3) * 8 + (i16 >> 2) + grp * 32) * S;
+#pragma unroll  // fully: the parameter pieces are indexed by u and must stay in registers
+        for (int u = 0; u < NUNIT; ++u) {
+            const int wu = wave + u * NWV, strip = wu % NSTRIP, c = wu / NSTRIP;
+            const unsigned char* q = src + strip * 128 * S + c * 8;
+            const s16x4 lo = lds_read_tr16(q), hi4 = lds_read_tr16(q + 4 * S);
+            const s16x8 t8 = {lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
+            long poff;
+            int left;
+            if (piece(u, poff, left)) {
+                const bf16x8 o = *(const bf16x8*)&t8;
+                if (pbf) fold_apply<bf16_t>((bf16_t*)pbase + poff, pv[u], o, pvec, left, g);
+                else fold_apply<float>((float*)pbase + poff, pv[u], o, pvec, left, g);
+            }
         }
         return;
     }
@@ -595,7 +654,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pipe_kernel(const GemmA
         }
     }
     WAIT_VM(0);  // the dummy loads of the last two tails must not land in the epilogue's tile
-    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN, EPI == EPI_BX_UPD>(g, tc, acc, smem);
+    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN, epi_fold_mode(EPI)>(g, tc, acc, smem);
     else epilogue<BM, BN, WGM, WGN, EPI, false>(g, tc, acc, smem);
 }
 
@@ -824,7 +883,7 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     if (!grp) __builtin_amdgcn_s_barrier();
     MUON_TRACE_STAMP(g, 2);
     WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
-    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN, EPI == EPI_BX_UPD>(g, tc, acc, smem);
+    if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN, epi_fold_mode(EPI)>(g, tc, acc, smem);
     else epilogue<BM, BN, WGM, WGN, EPI, true>(g, tc, acc, smem);
 }
 
@@ -926,6 +985,7 @@ hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t strea
             case EPI_SYMPOLY: return launch_pp_tail<EPI_SYMPOLY>(g, nblocks, rest, stream);
             case EPI_BX: return launch_pp_tail<EPI_BX>(g, nblocks, rest, stream);
             case EPI_BX_UPD: return launch_pp_tail<EPI_BX_UPD>(g, nblocks, rest, stream);
+            case EPI_BX_UPD_T: return launch_pp_tail<EPI_BX_UPD_T>(g, nblocks, rest, stream);
             default: return hipErrorInvalidValue;
         }
     }
@@ -934,6 +994,7 @@ hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t strea
         case EPI_SYMPOLY: return launch_cfg<EPI_SYMPOLY>(cfg, g, nblocks, stream);
         case EPI_BX: return launch_cfg<EPI_BX>(cfg, g, nblocks, stream);
         case EPI_BX_UPD: return launch_cfg<EPI_BX_UPD>(cfg, g, nblocks, stream);
+        case EPI_BX_UPD_T: return launch_cfg<EPI_BX_UPD_T>(cfg, g, nblocks, stream);
         default: return hipErrorInvalidValue;
     }
 }

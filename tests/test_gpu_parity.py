@@ -478,12 +478,14 @@ def test_grouped_equals_per_matrix_bitwise(env):
 
 
 @pytest.mark.parametrize("pdtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,cols,batch", [(256, 384, 3), (37, 53, 2), (100, 300, 2), (512, 1024, 2), (768, 2048, 3), (64, 64, 1)])
+@pytest.mark.parametrize("rows,cols,batch", [(256, 384, 3), (37, 53, 2), (100, 300, 2), (512, 1024, 2), (768, 2048, 3), (64, 64, 1),
+                                             (384, 256, 3), (53, 37, 2), (300, 100, 2), (1024, 512, 2), (2048, 768, 3), (1000, 520, 2)])
 def test_folded_update_equals_the_staged_sequence_bitwise(env, pdtype, rows, cols, batch):
-    """muon_hip_step_grouped lets the epilogue of the last B.X apply the scaled update to a parameter that has X's
-    orientation (rows <= cols), without writing the final X'.  The stage entry points run the same arithmetic through
-    the stand-alone update kernel (itself bit-identical to torch on the device): parameters and momentum must come out
-    equal bit for bit, ragged shapes and both parameter dtypes included."""
+    """muon_hip_step_grouped lets the epilogue of the last B.X apply the scaled update to the parameter without writing
+    the final X': directly when the parameter has X's orientation (rows <= cols), through a transposing gather out of
+    LDS when it is X's transpose (rows > cols).  The stage entry points run the same arithmetic through the stand-alone
+    update kernel (itself bit-identical to torch on the device): parameters and momentum must come out equal bit for
+    bit, ragged shapes, both orientations and both parameter dtypes included."""
     print(f"folded update {pdtype} {rows}x{cols} x{batch}", flush=True)
     lib, abi, mu, dev = env["lib"], env["abi"], env["mu"], env["dev"]
     gen = torch.Generator().manual_seed(rows * 13 + cols)
