@@ -455,6 +455,33 @@ def test_full_step_ragged_and_tall_shapes(env, dtype):
             assert wp <= 4e-3
 
 
+@pytest.mark.parametrize("hp", [
+    dict(lr=0.05, momentum=0.9, nesterov=False, weight_decay=0.0, ns_steps=5, rms_scale=True),
+    dict(lr=0.01, momentum=0.8, nesterov=True, weight_decay=0.1, ns_steps=1, rms_scale=True),
+    dict(lr=0.02, momentum=0.95, nesterov=True, weight_decay=0.01, ns_steps=3, rms_scale=False),
+    dict(lr=0.02, momentum=0.3, nesterov=False, weight_decay=0.01, ns_steps=4, rms_scale=False),
+    dict(lr=0.02, momentum=0.95, nesterov=True, weight_decay=0.01, ns_steps=0, rms_scale=False),
+], ids=lambda h: f"ns{h['ns_steps']}-{'nest' if h['nesterov'] else 'plain'}-{'rms' if h['rms_scale'] else 'ratio'}-b{h['momentum']}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_full_step_hyperparameters_against_the_oracle(env, hp, dtype):
+    """Every hyper-parameter of a Muon group away from the benchmark's value: no Nesterov blend, momentum below 0.5 (the
+    other branch of ATen's lerp), both scalings, no decay, 0 / 1 / 3 / 4 iterations (with none the update kernel runs,
+    otherwise the parameter is updated inside the last product), on wide, tall and ragged shapes, two steps each."""
+    names = ["wide", "tall", "square", "tall_ragged", "wide_ragged"]
+    shapes = [(128, 384), (384, 128), (256, 256), (210, 77), (90, 250)]
+    gen = torch.Generator().manual_seed(23)
+    weights = [(n, 0.02 * torch.randn(*s, generator=gen)) for n, s in zip(names, shapes)]
+    opt, orc, gp, cp = _build_opts(env, weights, hp, dtype, momentum_dtype=torch.float32 if dtype == torch.bfloat16 else None)
+    for step in range(2):
+        grads = [1e-3 * torch.randn(*s, generator=gen) for s in shapes]
+        wu, wm, wp = _check_step(opt, orc, gp, cp, grads, dtype, None, env=env)
+        print(f"hyper-parameters {hp} {dtype} step {step}: update {wu:.3e} momentum {wm:.3e} param {wp:.3e}", flush=True)
+        assert wm <= MOM_TOL
+        # fewer iterations leave less room for accumulation-order noise to grow; none is the rounded blend itself
+        assert wu <= (NS_TOL if hp["ns_steps"] >= 4 else 4e-3)
+        assert wp <= (2e-3 if dtype == torch.float32 else 4e-3) * max(1.0, hp["lr"] / 0.02) * (3.0 if hp["rms_scale"] else 1.0)
+
+
 def test_grouped_equals_per_matrix_bitwise(env):
     mu = env["mu"]
     weights, grads = make_param_set(dict(QWEN25_05B, q=(256, 256), o=(256, 256), k=(128, 256), v=(128, 256),
