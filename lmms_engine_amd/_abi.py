@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmuon_hip.so")
 
 F32, BF16 = 0, 1
-CFG_AUTO, CFG_128_PIPE, CFG_256_PIPE, CFG_256_PINGPONG, CFG_128_PINGPONG = -1, 0, 1, 2, 3
+CFG_AUTO, CFG_128_PIPE, CFG_256_PIPE, CFG_256_PINGPONG, CFG_128_PINGPONG, CFG_256_PERSIST = -1, 0, 1, 2, 3, 4
 GEMM_CONFIGS = list(range(4))
 K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW, K_ADAMW_MULTI, K_GRAD_NORM, K_CLIP_SCALE = range(10)
 KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw", "adamw_multi",

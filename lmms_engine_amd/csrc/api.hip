@@ -96,7 +96,9 @@ int pick_cfg(int M, int epi = EPI_BX, int kdim = 0) {
     (void)kdim;
     if (!use_tile256(M)) return GEMM_CFG_128_PINGPONG;
     if (epi != EPI_BX && M <= 512) return GEMM_CFG_128_PINGPONG;
-    return GEMM_CFG_256_PINGPONG;
+    // a.X + B.X walks its tiles in the persistent kernel (the launcher keeps the one-tile kernel for the launches that
+    // carry the parameter update and for those of at most one round); the symmetric products have no such kernel
+    return epi == EPI_BX ? GEMM_CFG_256_PERSIST : GEMM_CFG_256_PINGPONG;
 }
 
 int make_plan(int rows, int cols, int batch, Plan& p) {

@@ -14,7 +14,10 @@ enum {
     GEMM_CFG_256_PIPE = 1,      // 256x256 tile, 8 waves, the same pipeline
     GEMM_CFG_256_PINGPONG = 2,  // 256x256 tile, 8 waves in two alternating groups, four stages of 32 columns
     GEMM_CFG_128_PINGPONG = 3,  // 128x128 tile, the same eight-wave kernel, two workgroups per compute unit
-    GEMM_CFG_COUNT = 4
+    GEMM_CFG_256_PERSIST = 4,   // a.X + B.X: the ping-pong loop as a persistent kernel (a workgroup per compute unit walks
+                                // tiles, the next tile's first loads land behind the LDS-free epilogue); other products
+                                // and launches of at most one round run GEMM_CFG_256_PINGPONG
+    GEMM_CFG_COUNT = 5
 };
 
 struct GemmArgs {
@@ -43,6 +46,7 @@ struct GemmArgs {
     int upd_rows, upd_cols;       // the parameter's own (unpadded) shape
     float upd_scale, upd_decay, upd_alpha;  // python-double scale, 1 - lr*wd and -lr, as fp32
     int big_blocks;         // set by the launcher: workgroups that compute whole 256x256 tiles (split-tail kernel)
+    int ppx_slot;           // set by the launcher: which set of tile counters the persistent kernel uses
 #ifdef MUON_TILE_TRACE
     long* trace;            // measurement builds only: 8 longs per workgroup
 #endif

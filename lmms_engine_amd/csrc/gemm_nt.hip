@@ -473,6 +473,53 @@ __device__ __forceinline__ void epilogue_nn(const GemmArgs& g, const TileCoord& 
     }
 }
 
+// The same result for EPI_BX without LDS and without a barrier.  A lane holds, of fragment (i, j), columns 4q..4q+3
+// (q = lane / 16) of row lane % 16 as two packed registers.  v_permlane16_swap_b32 exchanges the odd 16-lane rows of
+// its first operand with the even rows of its second: applied to the registers of fragments j = 2t and 2t+1 it leaves
+// a lane of row 0 / 2 with columns 0..7 / 8..15 of fragment 2t and a lane of row 1 / 3 with those of fragment 2t+1,
+// i.e. 16 consecutive bytes of a row of X', and the 64 lanes of a wave with 16 rows x 64 bytes = one contiguous KB of
+// the blocked layout, the same store the LDS version issues.  The a.X pieces are loaded in the same pattern.
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
+    const bf16x2 p = {f2bf(a), f2bf(b)};
+    return *(const unsigned*)&p;
+}
+template <int BM, int BN, int WGM, int WGN>
+__device__ __forceinline__ void epilogue_nn_reg(const GemmArgs& g, const TileCoord& tc,
+                                                f32x4 (&acc)[BM / WGM / 16][BN / WGN / 16]) {
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 16, FN = WTN / 16;
+    static_assert(FN % 2 == 0 && BLK_COLS == 32, "a pair of fragments is one column block");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wm = wave / WGN, wn = wave % WGN, row = lane >> 4;
+    const int m0 = tc.ti * BM, n0 = tc.tj * BN;
+    // piece (i, t): row m0 + wm*WTM + 16 i + lane%16, columns n0 + wn*WTN + 32 t + 16 (row & 1) + 8 (row >> 1) .. + 7
+    const long lane_off = (long)((n0 >> BLK_SHIFT) + wn * (WTN / 32)) * BLK_ELEMS + (wm * WTM + (lane & 15)) * BLK_COLS +
+                          (row & 1) * 16 + (row >> 1) * 8;
+    const bf16_t* Et = g.Et + tc.bidx * g.strideEt + panel_offset(m0, g.cbEt) + lane_off;
+    bf16_t* C = g.C + tc.bidx * g.strideC + panel_offset(m0, g.cbC) + lane_off;
+    bf16x8 ev[FM][FN / 2];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int t = 0; t < FN / 2; ++t) ev[i][t] = *(const bf16x8*)(Et + i * 16 * BLK_COLS + (long)t * BLK_ELEMS);
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int t = 0; t < FN / 2; ++t) {
+            const f32x4 a = acc[i][2 * t], b = acc[i][2 * t + 1];
+            const u32x2v lo = __builtin_amdgcn_permlane16_swap(pack_bf16x2(a[0], a[1]), pack_bf16x2(b[0], b[1]), false, false);
+            const u32x2v hi = __builtin_amdgcn_permlane16_swap(pack_bf16x2(a[2], a[3]), pack_bf16x2(b[2], b[3]), false, false);
+            const u32x4 tw = {lo[0], hi[0], lo[1], hi[1]};
+            const bf16x8 tv = *(const bf16x8*)&tw;
+            bf16x8 o;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) o[k] = f2bf(rbf(g.s0 * bf2f(ev[i][t][k])) + bf2f(tv[k]));
+            *(bf16x8*)(C + i * 16 * BLK_COLS + (long)t * BLK_ELEMS) = o;
+        }
+}
+
 // Transposing LDS read of a Q fragment of BX: the stage holds the k-tile of X as pieces of 32 columns,
 // [piece][k][32 columns] with 64-byte rows, and a fragment is 16 columns x 32 k.  ds_read_b64_tr_b16 works in
 // groups of 16 lanes: lane j = 4r+s addresses row k+r, columns 4s..4s+3 of the group's 16 columns, and lane
@@ -882,6 +929,12 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     }
     if (!grp) __builtin_amdgcn_s_barrier();
     MUON_TRACE_STAMP(g, 2);
+    if constexpr (EPI == EPI_BX) {
+        // no LDS in this epilogue: the loads issued past the end may land while it runs (its own loads are behind
+        // them in the queue, so they have landed before the wave ends)
+        epilogue_nn_reg<BM, BN, WGM, WGN>(g, tc, acc);
+        return;
+    }
     WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
     if constexpr (QT) epilogue_nn<BM, BN, WGM, WGN, epi_fold_mode(EPI)>(g, tc, acc, smem);
     else epilogue<BM, BN, WGM, WGN, EPI, true>(g, tc, acc, smem);
@@ -913,6 +966,252 @@ __global__ void __launch_bounds__(512) gemm_nt_pp_tail_kernel(const GemmArgs g) 
         tc.tj = tc.tj * 2 + (quarter & 1);
         pp_tile<128, 128, 2, 4, EPI>(g, tc, smem);
     }
+}
+
+// ---- kernel 3: a.X + B.X as a persistent kernel ------------------------------------------------
+// The epilogue of EPI_BX needs no LDS (epilogue_nn_reg), so nothing stands between the k loops of two tiles: one
+// workgroup per compute unit walks tiles, the last three memory phases of a tile issue the first three k-tiles of the
+// workgroup's NEXT tile into the stages the current one has finished with, and they land while the waves drain their
+// accumulators.  What a one-tile workgroup pays around its k loop on top of the epilogue - the cold first loads (2 to
+// 3 us) and the hand-over of the compute unit to the next workgroup (2 to 3 us) - is a sixth of a tile when the
+// reduction is 24 k-tiles long (a 768-row expert matrix) and 4 % at 128.
+//
+// Tiles are handed out per XCD, in the order xcd_remap gives a one-tile-per-workgroup launch: workgroup b sits on
+// XCD b % 8 and takes "virtual workgroup ids" 8 n + b % 8.  Its first two n are static (b / 8 and b / 8 + grid / 8),
+// later ones come from an atomic counter of its XCD, asked for during the epilogue of the tile before the one whose
+// last phases need it.  The counters live in a file-scope array (zero when the library is loaded); the last
+// workgroup to leave puts the launch's slot back to zero, launches take slots in turn.
+constexpr int PPX_SLOTS = 64;
+struct PpxCounters {
+    unsigned next[XCD_COUNT][16];  // a cache line per XCD: tiles handed out beyond the two static rounds
+    unsigned done[16];             // workgroups that have left
+};
+__device__ PpxCounters g_ppx[PPX_SLOTS];
+
+#ifdef MUON_TILE_TRACE
+#define MUON_TRACE_STAMP_AT(g, idx, slot)                                                                          \
+    do {                                                                                                           \
+        if ((g).trace && threadIdx.x == 0) {                                                                       \
+            (g).trace[(long)(idx) * 8 + (slot)] = (long)__builtin_amdgcn_s_memrealtime();                          \
+            if ((slot) == 0) {                                                                                     \
+                (g).trace[(long)(idx) * 8 + 4] = (long)__builtin_amdgcn_s_memtime();                               \
+                (g).trace[(long)(idx) * 8 + 6] = (long)__builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)) | \
+                                                 ((long)__builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11)) << 32); \
+            }                                                                                                      \
+            if ((slot) == 3) (g).trace[(long)(idx) * 8 + 5] = (long)__builtin_amdgcn_s_memtime();                  \
+        }                                                                                                          \
+    } while (0)
+#else
+#define MUON_TRACE_STAMP_AT(g, idx, slot) do { } while (0)
+#endif
+
+__global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
+    constexpr int EPI = EPI_BX;
+    constexpr int BM = 256, BN = 256, WGM = 2, WGN = 4, NW = 8;
+    constexpr int BK4 = 32, ROWB = 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 16, FN = WTN / 16;
+    constexpr int A_BYTES = BM * ROWB, B_BYTES = BN * ROWB, STAGE = A_BYTES + B_BYTES;
+    constexpr int LA = BM / 16 / NW, LB = BN / 16 / NW;
+    constexpr int NLD = LA + LB;
+    constexpr int SLOT_OFF = 4 * STAGE;  // behind the four stages: where lane 0 leaves the next tile's id for the others
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int grp = wave >> 2;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int kb = g.kdim / BLK_COLS;
+    const int total = g.tiles_per_mat * g.batch;
+    const int grid = gridDim.x, xcd = blockIdx.x % XCD_COUNT;
+
+    auto panel_p = [&](const TileCoord& t) { return uniform_ptr(g.P + t.bidx * g.strideP + panel_offset(t.ti * BM, kb)); };
+    auto panel_q = [&](const TileCoord& t) {
+        return uniform_ptr(g.Q + t.bidx * g.strideQ + (long)(t.tj * BN >> BLK_SHIFT) * BLK_ELEMS);
+    };
+
+    // per-lane load offsets and LDS addresses: as in pp_tile
+    const int drow = lane >> 2;
+    const int dch = ((lane & 3) ^ pp_swizzle((lane >> 4) & 3)) * 8;
+    unsigned offa[LA], offb[LB];
+#pragma unroll
+    for (int n = 0; n < LA; ++n) offa[n] = (unsigned)(((wave * 16 * LA + n * 16 + drow) * BLK_COLS + dch) * 2);
+    const int qch = ((lane & 3) ^ (((drow >> 3) & 1) << 1)) * 8;
+#pragma unroll
+    for (int n = 0; n < LB; ++n) {
+        const int t = wave * LB + n;
+        offb[n] = (unsigned)(((t >> 1) * BLK_ELEMS + ((t & 1) * 16 + drow) * BLK_COLS + qch) * 2);
+    }
+    const int lds_a = wave * 16 * LA * ROWB;
+    const int lds_b = A_BYTES + wave * 16 * LB * ROWB;
+    const int nk = g.kdim / BK4;  // a multiple of 4, at least 8 (the launcher checks)
+
+    auto dma = [&](const char* base, unsigned voff, unsigned lds_byte) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_byte), "v"(voff), "s"(base)
+                     : "memory");
+    };
+    const unsigned lds_base = (unsigned)(uintptr_t)(lds_void_ptr)smem;
+    // k-tile kt of the tile whose panels are (P, Q), into stage kt & 3
+    auto issue_tile = [&](const bf16_t* P, const bf16_t* Q, int kt) {
+        const int k0 = kt * BK4;
+        const long koff = (long)(k0 >> BLK_SHIFT) * BLK_ELEMS + (k0 & (BLK_COLS - 1));
+        const char* ba = (const char*)(P + koff);
+        const char* bb = (const char*)(Q + (long)(k0 >> 8) * g.cbQ * BLK_ELEMS + (k0 & 255) * BLK_COLS);
+        const unsigned st = lds_base + (kt & 3) * STAGE;
+#pragma unroll
+        for (int n = 0; n < LA; ++n) dma(ba, offa[n], st + lds_a + n * 16 * ROWB);
+#pragma unroll
+        for (int n = 0; n < LB; ++n) dma(bb, offb[n], st + lds_b + n * 16 * ROWB);
+    };
+
+    const int sw = pp_swizzle((lane >> 2) & 3), kq = lane >> 4;
+    const int co = (kq ^ sw) << 4;
+    const int a_off = (wm * WTM + (lane & 15)) * ROWB + co;
+    const unsigned char* ra[2];
+    const unsigned char* rb[2][2];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        ra[half] = smem + half * 2 * STAGE + a_off;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+            rb[half][h] = smem + half * 2 * STAGE + A_BYTES + (wn * WTN / 32) * 2048 + qt_lane_offset(lane, h);
+    }
+
+    // this workgroup's tiles: the current one, the one after it (virtual ids; >= total means none)
+    int pid_cur = blockIdx.x, pid_nxt = blockIdx.x + grid;
+    TileCoord tc = tile_of<EPI>(g, xcd_remap(pid_cur, total));
+    const bf16_t* Pb = panel_p(tc);
+    const bf16_t* Qb = panel_q(tc);
+
+    MUON_TRACE_STAMP_AT(g, pid_cur, 0);
+    issue_tile(Pb, Qb, 0);
+    issue_tile(Pb, Qb, 1);
+    issue_tile(Pb, Qb, 2);
+    WAIT_VM(0);  // a tile starts with its k-tiles 0, 1 and 2 in LDS
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    MUON_TRACE_STAMP_AT(g, pid_cur, 1);
+    if (grp) __builtin_amdgcn_s_barrier();
+
+    for (;;) {
+        const bool has_next = pid_nxt < total;
+        // without a next tile the last phases load this tile's first k-tiles again, into stages nobody reads any more
+        const TileCoord ntc = has_next ? tile_of<EPI>(g, xcd_remap(pid_nxt, total)) : tc;
+        const bf16_t* Pn = panel_p(ntc);
+        const bf16_t* Qn = panel_q(ntc);
+
+        f32x4 acc[FM][FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+
+        // NEXT: the memory phase issues k-tile kt+3-nk of the next tile instead of k-tile kt+3 of this one.
+        // NOWAIT: the first two phases of a tile wait for no load: its k-tiles 0, 1 and 2 are in LDS when it starts
+        // (a count would make them wait for the stores of the epilogue before).
+        auto body = [&](int kt, auto stage_c, auto next_c, auto nowait_c) {
+            constexpr int SIDX = decltype(stage_c)::value;
+            constexpr bool NEXT = decltype(next_c)::value;
+            constexpr bool NOWAIT = decltype(nowait_c)::value;
+            bf16x8 fa[FM], fb[FN];
+#pragma unroll
+            for (int i = 0; i < FM; ++i) fa[i] = *(const bf16x8*)(ra[SIDX >> 1] + (SIDX & 1) * STAGE + i * 16 * ROWB);
+#pragma unroll
+            for (int j = 0; j < FN; ++j) fb[j] = lds_read_qt(rb[SIDX >> 1][j & 1] + (SIDX & 1) * STAGE + (j >> 1) * 2048);
+            if constexpr (NEXT) issue_tile(Pn, Qn, kt + 3 - nk);
+            else issue_tile(Pb, Qb, kt + 3);
+            WAIT_LGKM0();
+            if constexpr (!NOWAIT) WAIT_VM(2 * NLD);  // own loads of k-tile kt+1 have landed
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < FN; ++j)
+#pragma unroll
+                for (int i = 0; i < FM; ++i) acc[i][j] = mfma16(fb[j], fa[i], acc[i][j]);
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        using I2 = std::integral_constant<int, 2>;
+        using I3 = std::integral_constant<int, 3>;
+        using No = std::false_type;
+        using Yes = std::true_type;
+        body(0, I0{}, No{}, Yes{});
+        body(1, I1{}, No{}, Yes{});
+        body(2, I2{}, No{}, No{});
+        body(3, I3{}, No{}, No{});
+        for (int kt = 4; kt < nk - 4; kt += 4) {
+            body(kt, I0{}, No{}, No{});
+            body(kt + 1, I1{}, No{}, No{});
+            body(kt + 2, I2{}, No{}, No{});
+            body(kt + 3, I3{}, No{}, No{});
+        }
+        body(nk - 4, I0{}, No{}, No{});
+        body(nk - 3, I1{}, Yes{}, No{});
+        body(nk - 2, I2{}, Yes{}, No{});
+        body(nk - 1, I3{}, Yes{}, No{});
+        if (!grp) __builtin_amdgcn_s_barrier();  // the two groups leave the k loop together
+        MUON_TRACE_STAMP_AT(g, pid_cur, 2);
+
+        // Every wave drains its accumulators on its own.  One lane asks for the id of the tile after the next (an
+        // increment with wrap-around at 2^32 - 1: a plain atomicAdd of a uniform value is turned into a wave-wide
+        // reduction by the compiler, which then waits for the answer on the spot); the answer is needed at the end.
+        unsigned fetched = 0;
+        if (has_next && tid == 0) fetched = atomicInc(&g_ppx[g.ppx_slot].next[xcd][0], 0xffffffffu);
+        epilogue_nn_reg<BM, BN, WGM, WGN>(g, tc, acc);
+        // (the answer stays untouched until here: any arithmetic on it would be scheduled next to the atomic, with a
+        // wait for it)
+        asm volatile("" : "+v"(fetched));
+        if (tid == 0) *(int*)(smem + SLOT_OFF) = has_next ? (2 * (grid / XCD_COUNT) + (int)fetched) * XCD_COUNT + xcd : total;
+        // The loads of the epilogue are behind those of the next tile's first k-tiles in the queue and have been
+        // consumed, so every wave's share of those k-tiles has landed: publish them, and the id.
+        __syncthreads();
+        MUON_TRACE_STAMP_AT(g, pid_cur, 3);
+        if (!has_next) break;
+        pid_cur = pid_nxt;
+        pid_nxt = __builtin_amdgcn_readfirstlane(*(const int*)(smem + SLOT_OFF));
+        tc = ntc;
+        Pb = Pn;
+        Qb = Qn;
+        MUON_TRACE_STAMP_AT(g, pid_cur, 0);
+        MUON_TRACE_STAMP_AT(g, pid_cur, 1);
+        if (grp) __builtin_amdgcn_s_barrier();  // and enter the next tile a phase apart again
+    }
+    if (tid == 0) {
+        PpxCounters& c = g_ppx[g.ppx_slot];
+        // every workgroup has its last answer from `next` before it counts itself out, so the last one out may reset
+        if (atomicAdd(&c.done[0], 1u) == (unsigned)grid - 1) {
+            for (int x = 0; x < XCD_COUNT; ++x) atomicExch(&c.next[x][0], 0u);
+            atomicExch(&c.done[0], 0u);
+        }
+    }
+}
+
+std::atomic<unsigned> g_ppx_sequence{0};  // launches take the counter slots in turn
+
+hipError_t launch_ppx_bx(GemmArgs g, int nblocks, hipStream_t stream) {
+    constexpr int smem = 4 * (256 + 256) * 64 + 64;
+    static std::atomic<bool> configured{false};
+    if (!configured.load(std::memory_order_acquire)) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_ppx_bx_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return e;
+        configured.store(true, std::memory_order_release);
+    }
+    g.ppx_slot = (int)(g_ppx_sequence.fetch_add(1, std::memory_order_relaxed) % PPX_SLOTS);
+    const int grid = nblocks < GEMM_CU_COUNT ? nblocks : GEMM_CU_COUNT;
+    hipLaunchKernelGGL(gemm_nt_ppx_bx_kernel, dim3(grid), dim3(512), smem, stream, g);
+    return hipGetLastError();
 }
 
 template <int BM, int BN, int WGM, int WGN, int EPI, int FEED>
@@ -951,7 +1250,8 @@ int gemm_cfg_tile(int cfg) {
         case GEMM_CFG_128_PIPE:
         case GEMM_CFG_128_PINGPONG: return 128;
         case GEMM_CFG_256_PIPE:
-        case GEMM_CFG_256_PINGPONG: return 256;
+        case GEMM_CFG_256_PINGPONG:
+        case GEMM_CFG_256_PERSIST: return 256;
         default: return 0;
     }
 }
@@ -979,6 +1279,11 @@ hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t strea
     // Ping-pong kernel: split the tiles of a last round that would fill at most a quarter of the CUs (a 128x128
     // tile takes about 0.6 of the time of a 256x256 one, so one round of quarters beats a round of whole tiles).
     const int rest = nblocks % GEMM_CU_COUNT;
+    if (cfg == GEMM_CFG_256_PERSIST) {
+        // a.X + B.X with at least 8 k-tiles and more tiles than compute units; everything else takes the one-tile kernel
+        if (epi == EPI_BX && g.kdim >= 256 && nblocks > GEMM_CU_COUNT) return launch_ppx_bx(g, nblocks, stream);
+        cfg = GEMM_CFG_256_PINGPONG;
+    }
     if (cfg == GEMM_CFG_256_PINGPONG && nblocks > GEMM_CU_COUNT && rest > 0 && rest <= GEMM_CU_COUNT / 4) {
         switch (epi) {
             case EPI_SYRK: return launch_pp_tail<EPI_SYRK>(g, nblocks, rest, stream);

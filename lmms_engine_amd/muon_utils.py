@@ -128,6 +128,7 @@ def get_autotune_config():
         dict(BLOCK_SIZE_M=256, BLOCK_SIZE_N=256, BLOCK_SIZE_K=64, num_stages=2, num_warps=8, config=_abi.CFG_256_PIPE),
         dict(BLOCK_SIZE_M=256, BLOCK_SIZE_N=256, BLOCK_SIZE_K=32, num_stages=4, num_warps=8, config=_abi.CFG_256_PINGPONG),
         dict(BLOCK_SIZE_M=128, BLOCK_SIZE_N=128, BLOCK_SIZE_K=32, num_stages=4, num_warps=8, config=_abi.CFG_128_PINGPONG),
+        dict(BLOCK_SIZE_M=256, BLOCK_SIZE_N=256, BLOCK_SIZE_K=32, num_stages=4, num_warps=8, config=_abi.CFG_256_PERSIST),
     ]
 
 

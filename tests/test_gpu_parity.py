@@ -47,7 +47,7 @@ def _assert_product_close(got, ref64, absprod):
     assert not bad.any(), f"{int(bad.sum())} elements outside one bf16 ulp"
 
 
-CFGS = list(range(4))
+CFGS = list(range(5))
 
 
 def _pack(env, t):
@@ -188,6 +188,33 @@ def test_split_tail_is_bitwise_the_plain_kernel(env):
         abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, O.NS_COEFFS[0], cfg, 0))
         outs.append(_unpack(env, Xo, batch, M, K))
     assert torch.equal(outs[0], outs[1]) and not torch.isnan(outs[0]).any()
+
+
+def test_persistent_bx_is_bitwise_the_one_tile_kernel(env):
+    """The persistent configuration of a.X + B.X walks several tiles per workgroup (two static rounds, then tiles from
+    per-XCD counters), prefetches the next tile behind an epilogue that needs no LDS and re-uses its counters launch
+    after launch.  It adds the same products in the same order as the one-tile ping-pong kernel: X' must agree bit for
+    bit with the two-stage kernel (whose epilogue goes through LDS), on tile counts of exactly two rounds, of several
+    rounds, with a ragged last round, and with 8 k-tiles (the shortest reduction it takes); three launches in a row
+    (the counters must be back at zero)."""
+    lib, abi, dev, O = env["lib"], env["abi"], env["dev"], env["O"]
+    g = torch.Generator().manual_seed(78)
+    a_c = O.NS_COEFFS[0]
+    # rectangular tiles M/256 * K/256 per matrix: 512, 1280, 1320 (= 5 rounds + 40), 270 (= 1 round + 14), 768
+    for M, K, batch in ((512, 512, 128), (512, 1024, 160), (768, 2048, 55), (256, 256 * 27, 10), (1024, 256, 192)):
+        print(f"persistent vs one-tile: M={M} K={K} batch={batch}", flush=True)
+        Xb = _pack(env, (torch.randn(batch, M, K, generator=g) / 16).bfloat16().to(dev))
+        Bm = (torch.randn(batch, M, M, generator=g) / 16).bfloat16()
+        Bb = _pack(env, (torch.triu(Bm) + torch.triu(Bm, 1).mT).to(dev))
+        res = []
+        for cfg in (abi.CFG_256_PIPE, abi.CFG_256_PERSIST, abi.CFG_256_PERSIST, abi.CFG_256_PERSIST):
+            Xo = _blocked_nan(env, batch, M, K)
+            abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, a_c, cfg, 0))
+            torch.cuda.synchronize()
+            res.append(Xo.clone())
+        for rep in (1, 2, 3):
+            assert not torch.isnan(res[rep].float()).any(), rep
+            assert torch.equal(res[0], res[rep]), f"M={M} K={K} batch={batch}, launch {rep}"
 
 
 def test_gemm_entry_points_reject_bad_shapes(env):

@@ -119,7 +119,7 @@ def test_module_substitution_is_name_complete(monkeypatch):
     assert list(inspect.signature(mod.muon_update).parameters) == ["grad", "momentum", "beta", "ns_steps", "nesterov", "rms_scale"]
     assert list(inspect.signature(mod.apply_momentum).parameters) == ["grad", "momentum", "beta", "nesterov"]
     assert list(inspect.signature(mod.Muon.__init__).parameters)[:4] == ["self", "param_groups", "defaults", "is_deepspeed_enabled"]
-    assert len(mod.get_autotune_config()) == 4
+    assert len(mod.get_autotune_config()) == 5
 
 
 def test_keyword_semantics_are_announced_once(caplog):
