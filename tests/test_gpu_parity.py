@@ -533,7 +533,9 @@ def test_grouped_equals_per_matrix_bitwise(env):
 
 @pytest.mark.parametrize("pdtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,cols,batch", [(256, 384, 3), (37, 53, 2), (100, 300, 2), (512, 1024, 2), (768, 2048, 3), (64, 64, 1),
-                                             (384, 256, 3), (53, 37, 2), (300, 100, 2), (1024, 512, 2), (2048, 768, 3), (1000, 520, 2)])
+                                             (384, 256, 3), (53, 37, 2), (300, 100, 2), (1024, 512, 2), (2048, 768, 3), (1000, 520, 2),
+                                             # more tiles than compute units: the persistent kernel carries the update
+                                             (512, 1024, 40), (768, 2048, 24), (700, 1000, 30)])
 def test_folded_update_equals_the_staged_sequence_bitwise(env, pdtype, rows, cols, batch):
     """muon_hip_step_grouped lets the epilogue of the last B.X apply the scaled update to the parameter without writing
     the final X': directly when the parameter has X's orientation (rows <= cols), through a transposing gather out of
