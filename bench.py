@@ -450,8 +450,9 @@ def main():
     if "bx_axpy" in kernels:
         tot_ms, cnt = kern["bx_axpy"]
         achieved = bx_f * args.steps / (tot_ms * 1e-3) / 1e12
-        roofline = {"kernel": "gemm_nt_pp_kernel<256, 256, 2, 4, EPI_BX> (X' = a.X + B.X; the last of a step's five launches per "
-                              "chunk is EPI_BX_UPD, the same product with the parameter update in its epilogue)",
+        roofline = {"kernel": "X' = a.X + B.X: gemm_nt_ppx_bx_kernel (persistent, four of a step's five launches per chunk) and "
+                              "gemm_nt_pp_kernel<256, 256, 2, 4, EPI_BX_UPD | EPI_BX_UPD_T> (the last launch, the same product "
+                              "with the parameter update in its epilogue); all launches counted",
                     "bound": "mfma", "achieved": achieved,
                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                     "traffic": recorded_traffic(args.workload) if layers == w["layers"] else None,
