@@ -96,9 +96,11 @@ int pick_cfg(int M, int epi = EPI_BX, int kdim = 0) {
     (void)kdim;
     if (!use_tile256(M)) return GEMM_CFG_128_PINGPONG;
     if (epi != EPI_BX && M <= 512) return GEMM_CFG_128_PINGPONG;
-    // a.X + B.X walks its tiles in the persistent kernel (the launcher keeps the one-tile kernel for the launches that
-    // carry the parameter update and for those of at most one round); the symmetric products have no such kernel
-    return epi == EPI_BX ? GEMM_CFG_256_PERSIST : GEMM_CFG_256_PINGPONG;
+    // The persistent kernel where the launcher takes it: a.X + B.X, and the symmetric products with reductions of at
+    // most 2048 (past that a tile is long enough that what the persistent kernel removes around it no longer shows in
+    // a step that runs at the power limit); launches of at most one round of tiles and those that carry the parameter
+    // update run the one-tile ping-pong kernel.
+    return GEMM_CFG_256_PERSIST;
 }
 
 int make_plan(int rows, int cols, int batch, Plan& p) {

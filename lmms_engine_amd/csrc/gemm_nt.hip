@@ -520,6 +520,108 @@ __device__ __forceinline__ void epilogue_nn_reg(const GemmArgs& g, const TileCoo
         }
 }
 
+// Symmetric products without LDS and without a barrier.  A lane holds, of fragment (i, j), rows 4q..4q+3 (q = lane / 16)
+// of column lane % 16: 8-byte pieces of rows of the mirror image Ct, which leave exactly as the rows of X' above, with
+// fragments i = 2t and 2t+1 paired by v_permlane16_swap_b32 (SYMPOLY adds the b.A term to the paired pieces, read from
+// the mirror tile of A in the same pattern).  For the tile itself the finished values return to the fragment layout
+// (the swap is its own inverse) and every group of four lanes transposes its 4 x 4 elements in two exchanges:
+//   with the lane one away (DPP quad_perm [1,0,3,2]) the 16-bit halves of each register,
+//   with the lane two away (quad_perm [2,3,0,1]) one of the two registers,
+// after which lane 4a+s of row q holds columns 4a..4a+3 of row 4q+s of the fragment: 8-byte pieces of rows of C, a wave
+// store covering 16 rows x 32 bytes.  In a diagonal tile only the 32x32 blocks on or above the diagonal hold computed
+// values: they go out as Ct pieces (the lower half and the diagonal blocks) and, strictly above it, as C pieces.
+__device__ __forceinline__ void quad_transpose_b16(unsigned& p0, unsigned& p1, unsigned sel, bool upper) {
+    const unsigned t0 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)p0, 0xB1, 0xF, 0xF, false);
+    const unsigned t1 = (unsigned)__builtin_amdgcn_update_dpp(0, (int)p1, 0xB1, 0xF, 0xF, false);
+    p0 = __builtin_amdgcn_perm(t0, p0, sel);
+    p1 = __builtin_amdgcn_perm(t1, p1, sel);
+    const unsigned send = upper ? p0 : p1;
+    const unsigned recv = (unsigned)__builtin_amdgcn_update_dpp(0, (int)send, 0x4E, 0xF, 0xF, false);
+    p0 = upper ? recv : p0;
+    p1 = upper ? p1 : recv;
+}
+template <int BM, int BN, int WGM, int WGN, int EPI, unsigned MASK = 0>
+__device__ __forceinline__ void epilogue_sym_reg(const GemmArgs& g, const TileCoord& tc,
+                                                 f32x4 (&acc)[BM / WGM / 16][BN / WGN / 16]) {
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int FM = WTM / 16, FN = WTN / 16;
+    static_assert(FM % 2 == 0 && FN % 2 == 0 && BLK_COLS == 32, "a pair of fragments is one column block");
+    static_assert(EPI == EPI_SYRK || EPI == EPI_SYMPOLY, "symmetric products");
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int wm = wave / WGN, wn = wave % WGN, row = lane >> 4;
+    const int m0 = tc.ti * BM, n0 = tc.tj * BN;
+    const bool diag = tc.ti == tc.tj;
+    // Ct piece (t, j): row n0 + wn*WTN + 16 j + lane%16, columns m0 + wm*WTM + 32 t + 16 (row & 1) + 8 (row >> 1) .. + 7
+    const long ct_off = (long)((m0 >> BLK_SHIFT) + wm * (WTM / 32)) * BLK_ELEMS + (wn * WTN + (lane & 15)) * BLK_COLS +
+                        (row & 1) * 16 + (row >> 1) * 8;
+    bf16_t* Ct = g.Ct + tc.bidx * g.strideCt + panel_offset(n0, g.cbCt) + ct_off;
+    // C piece of fragment (i, j): row m0 + wm*WTM + 16 i + 4 row + lane%4, columns n0 + wn*WTN + 16 j + 4 (lane/4 % 4) .. + 3
+    bf16_t* C = g.C + tc.bidx * g.strideC + panel_offset(m0, g.cbC) + (long)((n0 >> BLK_SHIFT) + wn * (WTN / 32)) * BLK_ELEMS +
+                (wm * WTM + 4 * row + (lane & 3)) * BLK_COLS + ((lane >> 2) & 3) * 4;
+    const unsigned sel = (lane & 1) ? 0x03020706u : 0x05040100u;
+    const bool upper = (lane & 2) != 0;
+    // SYMPOLY: the b.A pieces of all but the last row of pairs are fetched up front, those of the last row once the
+    // first row is finished and its registers are free
+    bf16x8 ev[EPI == EPI_SYMPOLY ? FM / 2 : 1][EPI == EPI_SYMPOLY ? FN : 1];
+    const bf16_t* Et = g.Et + tc.bidx * g.strideEt + panel_offset(n0, g.cbEt) + ct_off;
+    constexpr int EV_LATE = FM / 2 > 2 ? FM / 2 - 1 : FM / 2;  // first row of pairs that is fetched late
+    auto load_ev = [&](int t) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) ev[t][j] = *(const bf16x8*)(Et + j * 16 * BLK_COLS + (long)t * BLK_ELEMS);
+    };
+    if constexpr (EPI == EPI_SYMPOLY) {
+#pragma unroll
+        for (int t = 0; t < EV_LATE; ++t) load_ev(t);
+    }
+    auto rounded = [&](float v) {
+        v = rbf(v);
+        if (EPI == EPI_SYMPOLY) v = g.s1 * v;
+        return v;
+    };
+#pragma unroll
+    for (int t = 0; t < FM / 2; ++t) {
+        if constexpr (EPI == EPI_SYMPOLY) {
+            if (t == 1 && EV_LATE < FM / 2) load_ev(EV_LATE);
+        }
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            // MASK: the fragments that this copy of a diagonal tile's loop has not computed (pp_skip_mask), known when
+            // the caller has one copy of the epilogue per mask; the test on the block indices covers the other callers
+            if ((MASK >> (2 * t * FN + j)) & 1) continue;
+            const int mblk = wm * (WTM / 32) + t, nblk = wn * (WTN / 32) + (j >> 1);
+            if (diag && mblk > nblk) continue;  // not computed: the mirror image of a block another wave holds
+            const f32x4 a = acc[2 * t][j], b = acc[2 * t + 1][j];
+            unsigned a01 = pack_bf16x2(rounded(a[0]), rounded(a[1])), a23 = pack_bf16x2(rounded(a[2]), rounded(a[3]));
+            unsigned b01 = pack_bf16x2(rounded(b[0]), rounded(b[1])), b23 = pack_bf16x2(rounded(b[2]), rounded(b[3]));
+            u32x2v lo = __builtin_amdgcn_permlane16_swap(a01, b01, false, false);
+            u32x2v hi = __builtin_amdgcn_permlane16_swap(a23, b23, false, false);
+            if constexpr (EPI == EPI_SYMPOLY) {
+                const u32x4 tw = {lo[0], hi[0], lo[1], hi[1]};
+                const bf16x8 tv = *(const bf16x8*)&tw;
+                bf16x8 o;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) o[k] = f2bf(rbf(g.s0 * bf2f(ev[t][j][k])) + bf2f(tv[k]));
+                *(bf16x8*)(Ct + j * 16 * BLK_COLS + (long)t * BLK_ELEMS) = o;
+                if (diag && mblk == nblk) continue;
+                const u32x4 ow = *(const u32x4*)&o;
+                lo = __builtin_amdgcn_permlane16_swap(ow[0], ow[2], false, false);
+                hi = __builtin_amdgcn_permlane16_swap(ow[1], ow[3], false, false);
+                a01 = lo[0], b01 = lo[1], a23 = hi[0], b23 = hi[1];
+            } else {
+                const u32x4 tw = {lo[0], hi[0], lo[1], hi[1]};
+                *(u32x4*)(Ct + j * 16 * BLK_COLS + (long)t * BLK_ELEMS) = tw;
+                if (diag && mblk == nblk) continue;
+            }
+            quad_transpose_b16(a01, a23, sel, upper);
+            quad_transpose_b16(b01, b23, sel, upper);
+            bf16_t* cp = C + (2 * t) * 16 * BLK_COLS + (long)(j >> 1) * BLK_ELEMS + (j & 1) * 16;
+            *(u32x2v*)cp = u32x2v{a01, a23};
+            *(u32x2v*)(cp + 16 * BLK_COLS) = u32x2v{b01, b23};
+        }
+    }
+}
+
 // Transposing LDS read of a Q fragment of BX: the stage holds the k-tile of X as pieces of 32 columns,
 // [piece][k][32 columns] with 64-byte rows, and a fragment is 16 columns x 32 k.  ds_read_b64_tr_b16 works in
 // groups of 16 lanes: lane j = 4r+s addresses row k+r, columns 4s..4s+3 of the group's 16 columns, and lane
@@ -885,7 +987,8 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
 #pragma unroll
         for (int j = 0; j < FN; ++j)
 #pragma unroll
-            for (int i = 0; i < FM; ++i) {
+            for (int ii = 0; ii < FM; ++ii) {
+                const int i = (j & 1) ? FM - 1 - ii : ii;
                 if (QT)  // operands swapped: a lane then holds 4 consecutive columns of one row of the tile
                     acc[i][j] = mfma16(fb[j], fa[i], acc[i][j]);
                 else if (kept(i, j))
@@ -933,6 +1036,11 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
         // no LDS in this epilogue: the loads issued past the end may land while it runs (its own loads are behind
         // them in the queue, so they have landed before the wave ends)
         epilogue_nn_reg<BM, BN, WGM, WGN>(g, tc, acc);
+        return;
+    }
+    if constexpr (EPI == EPI_SYMPOLY && BM == 256) {
+        // measured: without LDS b.A + c.A.A is 0.5 % faster on whole 256-tiles, X.Xt 0.6 % slower
+        epilogue_sym_reg<BM, BN, WGM, WGN, EPI>(g, tc, acc);
         return;
     }
     WAIT_VM(0);  // the loads issued past the end must not land in the epilogue's tile
@@ -1005,8 +1113,10 @@ __device__ PpxCounters g_ppx[PPX_SLOTS];
 #define MUON_TRACE_STAMP_AT(g, idx, slot) do { } while (0)
 #endif
 
-__global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
-    constexpr int EPI = EPI_BX;
+template <int EPI>
+__global__ void __launch_bounds__(512) gemm_nt_ppx_kernel(const GemmArgs g) {
+    static_assert(EPI == EPI_BX || EPI == EPI_SYRK || EPI == EPI_SYMPOLY, "the epilogues that need no LDS");
+    constexpr bool QT = EPI == EPI_BX;  // Q is X itself, rows = reduction index
     constexpr int BM = 256, BN = 256, WGM = 2, WGN = 4, NW = 8;
     constexpr int BK4 = 32, ROWB = 64;
     constexpr int WTM = BM / WGM, WTN = BN / WGN;
@@ -1027,7 +1137,8 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
 
     auto panel_p = [&](const TileCoord& t) { return uniform_ptr(g.P + t.bidx * g.strideP + panel_offset(t.ti * BM, kb)); };
     auto panel_q = [&](const TileCoord& t) {
-        return uniform_ptr(g.Q + t.bidx * g.strideQ + (long)(t.tj * BN >> BLK_SHIFT) * BLK_ELEMS);
+        return uniform_ptr(g.Q + t.bidx * g.strideQ +
+                           (QT ? (long)(t.tj * BN >> BLK_SHIFT) * BLK_ELEMS : panel_offset(t.tj * BN, kb)));
     };
 
     // per-lane load offsets and LDS addresses: as in pp_tile
@@ -1040,7 +1151,8 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
 #pragma unroll
     for (int n = 0; n < LB; ++n) {
         const int t = wave * LB + n;
-        offb[n] = (unsigned)(((t >> 1) * BLK_ELEMS + ((t & 1) * 16 + drow) * BLK_COLS + qch) * 2);
+        offb[n] = QT ? (unsigned)(((t >> 1) * BLK_ELEMS + ((t & 1) * 16 + drow) * BLK_COLS + qch) * 2)
+                     : (unsigned)(((wave * 16 * LB + n * 16 + drow) * BLK_COLS + dch) * 2);
     }
     const int lds_a = wave * 16 * LA * ROWB;
     const int lds_b = A_BYTES + wave * 16 * LB * ROWB;
@@ -1058,7 +1170,7 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
         const int k0 = kt * BK4;
         const long koff = (long)(k0 >> BLK_SHIFT) * BLK_ELEMS + (k0 & (BLK_COLS - 1));
         const char* ba = (const char*)(P + koff);
-        const char* bb = (const char*)(Q + (long)(k0 >> 8) * g.cbQ * BLK_ELEMS + (k0 & 255) * BLK_COLS);
+        const char* bb = (const char*)(Q + (QT ? (long)(k0 >> 8) * g.cbQ * BLK_ELEMS + (k0 & 255) * BLK_COLS : koff));
         const unsigned st = lds_base + (kt & 3) * STAGE;
 #pragma unroll
         for (int n = 0; n < LA; ++n) dma(ba, offa[n], st + lds_a + n * 16 * ROWB);
@@ -1069,6 +1181,7 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
     const int sw = pp_swizzle((lane >> 2) & 3), kq = lane >> 4;
     const int co = (kq ^ sw) << 4;
     const int a_off = (wm * WTM + (lane & 15)) * ROWB + co;
+    const int b_off = A_BYTES + (wn * WTN + (lane & 15)) * ROWB + co;
     const unsigned char* ra[2];
     const unsigned char* rb[2][2];
 #pragma unroll
@@ -1076,7 +1189,8 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
         ra[half] = smem + half * 2 * STAGE + a_off;
 #pragma unroll
         for (int h = 0; h < 2; ++h)
-            rb[half][h] = smem + half * 2 * STAGE + A_BYTES + (wn * WTN / 32) * 2048 + qt_lane_offset(lane, h);
+            rb[half][h] = QT ? smem + half * 2 * STAGE + A_BYTES + (wn * WTN / 32) * 2048 + qt_lane_offset(lane, h)
+                             : smem + half * 2 * STAGE + b_off;
     }
 
     // this workgroup's tiles: the current one, the one after it (virtual ids; >= total means none)
@@ -1102,26 +1216,40 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
         const bf16_t* Pn = panel_p(ntc);
         const bf16_t* Qn = panel_q(ntc);
 
-        f32x4 acc[FM][FN];
-#pragma unroll
-        for (int i = 0; i < FM; ++i)
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+        const bool diag = !QT && tc.ti == tc.tj;
+        unsigned fetched = 0;
+        // One tile, k loop and epilogue, for the waves whose skip mask in a diagonal tile is `mask_c` (pp_tile): a copy of
+        // its own per mask, each with its own accumulators from the first MFMA to the last store.
+        auto run_tile = [&](auto mask_c) {
+        f32x4 acc[FM][FN];  // defined by the MFMAs of the tile's first k-tile, which add to zero
 
         // NEXT: the memory phase issues k-tile kt+3-nk of the next tile instead of k-tile kt+3 of this one.
         // NOWAIT: the first two phases of a tile wait for no load: its k-tiles 0, 1 and 2 are in LDS when it starts
         // (a count would make them wait for the stores of the epilogue before).
-        auto body = [&](int kt, auto stage_c, auto next_c, auto nowait_c) {
+        constexpr unsigned MASK = decltype(mask_c)::value;  // fragments a wave skips in a diagonal tile
+        auto body = [&](int kt, auto stage_c, auto next_c, auto nowait_c, auto first_c) {
             constexpr int SIDX = decltype(stage_c)::value;
             constexpr bool NEXT = decltype(next_c)::value;
             constexpr bool NOWAIT = decltype(nowait_c)::value;
+            constexpr bool FIRST = decltype(first_c)::value;
+            auto kept = [](int i, int j) { return !((MASK >> (i * FN + j)) & 1); };
             bf16x8 fa[FM], fb[FN];
 #pragma unroll
-            for (int i = 0; i < FM; ++i) fa[i] = *(const bf16x8*)(ra[SIDX >> 1] + (SIDX & 1) * STAGE + i * 16 * ROWB);
+            for (int i = 0; i < FM; ++i) {
+                bool used = false;
 #pragma unroll
-            for (int j = 0; j < FN; ++j) fb[j] = lds_read_qt(rb[SIDX >> 1][j & 1] + (SIDX & 1) * STAGE + (j >> 1) * 2048);
+                for (int j = 0; j < FN; ++j) used |= kept(i, j);
+                if (used) fa[i] = *(const bf16x8*)(ra[SIDX >> 1] + (SIDX & 1) * STAGE + i * 16 * ROWB);
+            }
+#pragma unroll
+            for (int j = 0; j < FN; ++j) {
+                bool used = false;
+#pragma unroll
+                for (int i = 0; i < FM; ++i) used |= kept(i, j);
+                if (!used) continue;
+                if (QT) fb[j] = lds_read_qt(rb[SIDX >> 1][j & 1] + (SIDX & 1) * STAGE + (j >> 1) * 2048);
+                else fb[j] = *(const bf16x8*)(rb[SIDX >> 1][0] + (SIDX & 1) * STAGE + j * 16 * ROWB);
+            }
             if constexpr (NEXT) issue_tile(Pn, Qn, kt + 3 - nk);
             else issue_tile(Pb, Qb, kt + 3);
             WAIT_LGKM0();
@@ -1134,7 +1262,12 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
 #pragma unroll
             for (int j = 0; j < FN; ++j)
 #pragma unroll
-                for (int i = 0; i < FM; ++i) acc[i][j] = mfma16(fb[j], fa[i], acc[i][j]);
+                for (int ii = 0; ii < FM; ++ii) {
+                    const int i = (j & 1) ? FM - 1 - ii : ii;  // back and forth: consecutive MFMAs share an operand
+                    const f32x4 c = FIRST ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[i][j];
+                    if (QT) acc[i][j] = mfma16(fb[j], fa[i], c);
+                    else if (kept(i, j)) acc[i][j] = mfma16(fa[i], fb[j], c);
+                }
             __builtin_amdgcn_sched_barrier(0);
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_barrier();
@@ -1147,29 +1280,60 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
         using I3 = std::integral_constant<int, 3>;
         using No = std::false_type;
         using Yes = std::true_type;
-        body(0, I0{}, No{}, Yes{});
-        body(1, I1{}, No{}, Yes{});
-        body(2, I2{}, No{}, No{});
-        body(3, I3{}, No{}, No{});
+        body(0, I0{}, No{}, Yes{}, Yes{});
+        body(1, I1{}, No{}, Yes{}, No{});
+        body(2, I2{}, No{}, No{}, No{});
+        body(3, I3{}, No{}, No{}, No{});
         for (int kt = 4; kt < nk - 4; kt += 4) {
-            body(kt, I0{}, No{}, No{});
-            body(kt + 1, I1{}, No{}, No{});
-            body(kt + 2, I2{}, No{}, No{});
-            body(kt + 3, I3{}, No{}, No{});
+            body(kt, I0{}, No{}, No{}, No{});
+            body(kt + 1, I1{}, No{}, No{}, No{});
+            body(kt + 2, I2{}, No{}, No{}, No{});
+            body(kt + 3, I3{}, No{}, No{}, No{});
         }
-        body(nk - 4, I0{}, No{}, No{});
-        body(nk - 3, I1{}, Yes{}, No{});
-        body(nk - 2, I2{}, Yes{}, No{});
-        body(nk - 1, I3{}, Yes{}, No{});
+        body(nk - 4, I0{}, No{}, No{}, No{});
+        body(nk - 3, I1{}, Yes{}, No{}, No{});
+        body(nk - 2, I2{}, Yes{}, No{}, No{});
+        body(nk - 1, I3{}, Yes{}, No{}, No{});
         if (!grp) __builtin_amdgcn_s_barrier();  // the two groups leave the k loop together
         MUON_TRACE_STAMP_AT(g, pid_cur, 2);
 
         // Every wave drains its accumulators on its own.  One lane asks for the id of the tile after the next (an
         // increment with wrap-around at 2^32 - 1: a plain atomicAdd of a uniform value is turned into a wave-wide
         // reduction by the compiler, which then waits for the answer on the spot); the answer is needed at the end.
-        unsigned fetched = 0;
         if (has_next && tid == 0) fetched = atomicInc(&g_ppx[g.ppx_slot].next[xcd][0], 0xffffffffu);
-        epilogue_nn_reg<BM, BN, WGM, WGN>(g, tc, acc);
+        if constexpr (QT) {
+            epilogue_nn_reg<BM, BN, WGM, WGN>(g, tc, acc);
+        } else {
+            epilogue_sym_reg<BM, BN, WGM, WGN, EPI, MASK>(g, tc, acc);
+            // What says that this wave's share of the next tile's first k-tiles has landed: B.X and b.A + c.A.A consume
+            // loads that were issued after them (the queue returns in order).  X.Xt loads nothing, and in a diagonal
+            // tile a wave may have nothing to finish at all: there the count is explicit (48 stores went out after the
+            // loads off the diagonal, an unknown number on it).
+            asm volatile("" ::: "memory");
+            if (diag) WAIT_VM(0);
+            else if (EPI == EPI_SYRK) WAIT_VM(FM * FN / 2 * 3);
+            asm volatile("" ::: "memory");
+        }
+        };  // run_tile
+        if (!diag) {
+            run_tile(std::integral_constant<unsigned, 0>{});
+        } else {
+            auto run_if_mine = [&](auto wave_c) {
+                constexpr int W = decltype(wave_c)::value;
+                constexpr unsigned M = pp_skip_mask<WTM, WTN, FM, FN, WGN>(W);
+                if constexpr (pp_first_with_mask<WTM, WTN, FM, FN, WGN>(W)) {
+                    if (pp_skip_mask<WTM, WTN, FM, FN, WGN>(wave) == M) run_tile(std::integral_constant<unsigned, M>{});
+                }
+            };
+            run_if_mine(std::integral_constant<int, 0>{});
+            run_if_mine(std::integral_constant<int, 1>{});
+            run_if_mine(std::integral_constant<int, 2>{});
+            run_if_mine(std::integral_constant<int, 3>{});
+            run_if_mine(std::integral_constant<int, 4>{});
+            run_if_mine(std::integral_constant<int, 5>{});
+            run_if_mine(std::integral_constant<int, 6>{});
+            run_if_mine(std::integral_constant<int, 7>{});
+        }
         // (the answer stays untouched until here: any arithmetic on it would be scheduled next to the atomic, with a
         // wait for it)
         asm volatile("" : "+v"(fetched));
@@ -1200,17 +1364,18 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_bx_kernel(const GemmArgs g) {
 
 std::atomic<unsigned> g_ppx_sequence{0};  // launches take the counter slots in turn
 
-hipError_t launch_ppx_bx(GemmArgs g, int nblocks, hipStream_t stream) {
+template <int EPI>
+hipError_t launch_ppx(GemmArgs g, int nblocks, hipStream_t stream) {
     constexpr int smem = 4 * (256 + 256) * 64 + 64;
-    static std::atomic<bool> configured{false};
+    static std::atomic<bool> configured{false};  // per instantiation
     if (!configured.load(std::memory_order_acquire)) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_ppx_bx_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_ppx_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
         configured.store(true, std::memory_order_release);
     }
     g.ppx_slot = (int)(g_ppx_sequence.fetch_add(1, std::memory_order_relaxed) % PPX_SLOTS);
     const int grid = nblocks < GEMM_CU_COUNT ? nblocks : GEMM_CU_COUNT;
-    hipLaunchKernelGGL(gemm_nt_ppx_bx_kernel, dim3(grid), dim3(512), smem, stream, g);
+    hipLaunchKernelGGL(gemm_nt_ppx_kernel<EPI>, dim3(grid), dim3(512), smem, stream, g);
     return hipGetLastError();
 }
 
@@ -1273,6 +1438,12 @@ hipError_t launch_pp_tail(GemmArgs g, int nblocks, int rest, hipStream_t stream)
     return hipGetLastError();
 }
 
+#ifndef PPX_SYRK_MAXK
+#define PPX_SYRK_MAXK 2048
+#endif
+#ifndef PPX_SYMPOLY_MAXK
+#define PPX_SYMPOLY_MAXK 2048
+#endif
 hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t stream) {
     const int nblocks = g.tiles_per_mat * g.batch;
     if (nblocks <= 0) return hipSuccess;
@@ -1281,7 +1452,11 @@ hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t strea
     const int rest = nblocks % GEMM_CU_COUNT;
     if (cfg == GEMM_CFG_256_PERSIST) {
         // a.X + B.X with at least 8 k-tiles and more tiles than compute units; everything else takes the one-tile kernel
-        if (epi == EPI_BX && g.kdim >= 256 && nblocks > GEMM_CU_COUNT) return launch_ppx_bx(g, nblocks, stream);
+        if (g.kdim >= 256 && nblocks > GEMM_CU_COUNT) {
+            if (epi == EPI_BX) return launch_ppx<EPI_BX>(g, nblocks, stream);
+            if (epi == EPI_SYRK && g.kdim <= PPX_SYRK_MAXK) return launch_ppx<EPI_SYRK>(g, nblocks, stream);
+            if (epi == EPI_SYMPOLY && g.kdim <= PPX_SYMPOLY_MAXK) return launch_ppx<EPI_SYMPOLY>(g, nblocks, stream);
+        }
         cfg = GEMM_CFG_256_PINGPONG;
     }
     if (cfg == GEMM_CFG_256_PINGPONG && nblocks > GEMM_CU_COUNT && rest > 0 && rest <= GEMM_CU_COUNT / 4) {

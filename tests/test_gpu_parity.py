@@ -217,6 +217,35 @@ def test_persistent_bx_is_bitwise_the_one_tile_kernel(env):
             assert torch.equal(res[0], res[rep]), f"M={M} K={K} batch={batch}, launch {rep}"
 
 
+def test_persistent_symmetric_products_are_bitwise_the_two_stage_kernel(env):
+    """X.Xt and b.A + c.A.A with reductions of at most 2048 run in the persistent kernel when a launch has more tiles
+    than compute units: triangular tile lists, diagonal tiles in which every wave skips the fragments below the
+    diagonal, and an epilogue that transposes in registers instead of LDS.  Both outputs must agree bit for bit with
+    the two-stage kernel (whole diagonal tiles, epilogue through LDS) and with the one-tile ping-pong kernel, be symmetric
+    bit for bit, and stay so on three launches in a row; tile counts with a ragged last round, 8 k-tiles (the shortest reduction) and 64 (the longest)."""
+    lib, abi, dev, O = env["lib"], env["abi"], env["dev"], env["O"]
+    g = torch.Generator().manual_seed(79)
+    _, b_c, c_c = O.NS_COEFFS
+    # triangular tiles T(T+1)/2 per matrix with T = M/256: 330, 300, 300, 288, 280
+    for M, K, batch in ((768, 2048, 55), (512, 256, 100), (1024, 1024, 30), (2048, 512, 8), (1792, 1280, 10)):
+        print(f"persistent symmetric vs two-stage: M={M} K={K} batch={batch}", flush=True)
+        Xb = _pack(env, (torch.randn(batch, M, K, generator=g) / 16).bfloat16().to(dev))
+        res = []
+        for cfg in (abi.CFG_256_PIPE, abi.CFG_256_PINGPONG, abi.CFG_256_PERSIST, abi.CFG_256_PERSIST, abi.CFG_256_PERSIST):
+            A = _blocked_nan(env, batch, M, M)
+            B = _blocked_nan(env, batch, M, M)
+            abi.check(lib.muon_hip_syrk_bf16(Xb.data_ptr(), A.data_ptr(), M, K, batch, cfg, 0))
+            abi.check(lib.muon_hip_sympoly_bf16(A.data_ptr(), B.data_ptr(), M, batch, b_c, c_c, cfg, 0))
+            torch.cuda.synchronize()
+            res.append((A.clone(), B.clone()))
+        for rep in (1, 2, 3, 4):  # the one-tile ping-pong kernel, then the persistent one three times
+            for name, ref, got in (("syrk", res[0][0], res[rep][0]), ("sympoly", res[0][1], res[rep][1])):
+                assert not torch.isnan(got.float()).any(), (name, rep)
+                assert torch.equal(ref, got), f"{name} M={M} K={K} batch={batch}, launch {rep}"
+        Bd = _unpack(env, res[1][1], batch, M, M)
+        assert torch.equal(Bd, Bd.mT.contiguous())
+
+
 def test_gemm_entry_points_reject_bad_shapes(env):
     lib, abi = env["lib"], env["abi"]
     x = torch.zeros(256 * 256, dtype=torch.bfloat16, device=env["dev"])
