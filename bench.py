@@ -7,9 +7,11 @@ lr 0.02, momentum 0.95 Nesterov, wd 0.01, 5 NS steps) with everything resident i
 prints ONE JSON line.  `value` is the algorithmic Newton-Schulz FLOPs of one step,
 steps*(3 M^2 K + M^3) per matrix, divided by the whole step time.
 
-The `roofline` object is for the dominant kernel (the B.X GEMM with the a.X epilogue): its
-algorithmic FLOPs per launch over its mean launch time, measured with HIP events recorded
-around every launch inside the timed region, against the dense bf16 MFMA peak.
+The `roofline` object is for the dominant kernel (the persistent B.X GEMM with the a.X epilogue,
+two fifths of the step): its algorithmic FLOPs per launch over its mean launch time, measured with
+HIP events recorded around every launch inside the timed region, against the dense bf16 MFMA peak.
+The one B.X launch in five that carries the parameter update is another kernel and has its own
+entry under `kernels`.
 `cpu_baseline` times the CPU oracle (a torch restatement of the reference step, test
 infrastructure) on one matrix per shape bucket and scales by the bucket counts.
 """
@@ -45,7 +47,7 @@ def git_blob_hash(path):
 
 
 def recorded_traffic(workload):
-    """bytes per B.X launch from the tracked counter summary, or None when absent or measured on other code."""
+    """bytes per launch of the persistent B.X kernel from the tracked counter summary, or None when absent or measured on other code."""
     try:
         cur = git_blob_hash(GEMM_SOURCE)
         for line in open(TRAFFIC_SUMMARY):
@@ -429,7 +431,12 @@ def main():
     # With at least one iteration the parameters are updated by the epilogue of the last B.X of the step (its time is
     # inside bx_axpy) and the update kernel does not run: it appears below only if it was launched.
     upd_elements = elements
-    work = {"syrk": (syrk_f, "flop"), "sympoly": (symp_f, "flop"), "bx_axpy": (bx_f, "flop"),
+    # The launch that carries the update (one of the ns_steps B.X launches of every chunk) is timed on its own: it is
+    # another kernel, with the parameter's bytes in its epilogue.
+    folded = kern.get("bx_axpy_update", (0.0, 0))[1] > 0
+    bx_plain_f = bx_f * (HP["ns_steps"] - 1) / HP["ns_steps"] if folded else bx_f
+    work = {"syrk": (syrk_f, "flop"), "sympoly": (symp_f, "flop"), "bx_axpy": (bx_plain_f, "flop"),
+            "bx_axpy_update": (bx_f - bx_plain_f, "flop"),
             "momentum_norm": (mom_bytes, "byte"), "normalize": (elements * 4, "byte"),
             "apply_update": (upd_elements * (2 + 2 * gb), "byte")}
     kernels = {}
@@ -449,16 +456,16 @@ def main():
     roofline = None
     if "bx_axpy" in kernels:
         tot_ms, cnt = kern["bx_axpy"]
-        achieved = bx_f * args.steps / (tot_ms * 1e-3) / 1e12
-        roofline = {"kernel": "X' = a.X + B.X: gemm_nt_ppx_bx_kernel (persistent, four of a step's five launches per chunk) and "
-                              "gemm_nt_pp_kernel<256, 256, 2, 4, EPI_BX_UPD | EPI_BX_UPD_T> (the last launch, the same product "
-                              "with the parameter update in its epilogue); all launches counted",
+        achieved = bx_plain_f * args.steps / (tot_ms * 1e-3) / 1e12
+        roofline = {"kernel": "gemm_nt_ppx_kernel<EPI_BX>: X' = a.X + B.X, the persistent kernel (the first ns_steps - 1 of the "
+                              "B.X launches of every chunk; the last one, which carries the parameter update in its "
+                              "epilogue, is another kernel: kernels.bx_axpy_update)",
                     "bound": "mfma", "achieved": achieved,
                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                     "traffic": recorded_traffic(args.workload) if layers == w["layers"] else None,
                     "launches": cnt, "avg_launch_ms": tot_ms / cnt,
-                    "algorithmic_flop_per_launch": bx_f * args.steps / cnt}
-    gemm_ms = sum(kernels[k]["ms_per_step"] for k in ("syrk", "sympoly", "bx_axpy") if k in kernels)
+                    "algorithmic_flop_per_launch": bx_plain_f * args.steps / cnt}
+    gemm_ms = sum(kernels[k]["ms_per_step"] for k in ("syrk", "sympoly", "bx_axpy", "bx_axpy_update") if k in kernels)
 
     out = {
         "metric": METRIC,

@@ -48,7 +48,8 @@ extern "C" {
 #define MUON_HIP_K_ADAMW_MULTI 7
 #define MUON_HIP_K_GRAD_NORM 8
 #define MUON_HIP_K_CLIP_SCALE 9
-#define MUON_HIP_K_COUNT 10
+#define MUON_HIP_K_BX_UPDATE 10 /* the a.X + B.X launch that carries the parameter update in its epilogue */
+#define MUON_HIP_K_COUNT 11
 
 /* GEMM kernel variants; MUON_HIP_CFG_AUTO picks per kernel and shape.  All feed LDS with direct
  * global->LDS loads (global_load_lds_dwordx4), software pipelined behind the MFMAs. */

@@ -19,7 +19,7 @@ CFG_AUTO, CFG_128_PIPE, CFG_256_PIPE, CFG_256_PINGPONG, CFG_128_PINGPONG, CFG_25
 GEMM_CONFIGS = list(range(4))
 K_MOMENTUM, K_NORMALIZE, K_SYRK, K_SYMPOLY, K_BX, K_UPDATE, K_ADAMW, K_ADAMW_MULTI, K_GRAD_NORM, K_CLIP_SCALE = range(10)
 KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "apply_update", "adamw", "adamw_multi",
-                "grad_norm", "clip_scale"]
+                "grad_norm", "clip_scale", "bx_axpy_update"]
 MULTI_CHUNK = 16384  # MUON_HIP_MULTI_CHUNK
 STATIC_MAX_CHUNKS = 1 << 20  # MUON_HIP_STATIC_MAX_CHUNKS
 PROBE_OPERAND_BYTES, PROBE_SINK_FLOATS = 256 * 12 * 512 * 16, 256 * 512  # MUON_HIP_PROBE_*

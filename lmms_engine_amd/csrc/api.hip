@@ -247,7 +247,7 @@ int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int K
         g.upd_alpha = (float)(-fold->lr);
     }
     SET_TRACE(g);
-    Timed t(MUON_HIP_K_BX, s);
+    Timed t(fold ? MUON_HIP_K_BX_UPDATE : MUON_HIP_K_BX, s);
     hipError_t e = launch_gemm_nt(cfg, !fold ? EPI_BX : fold->rows <= fold->cols ? EPI_BX_UPD : EPI_BX_UPD_T, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "bx launch");
 }
