@@ -275,6 +275,28 @@ def test_newton_schulz_small_shapes(env, rows, cols):
         assert rel_fro(mu.fast_newtonschulz(G.to(env["dev"]), steps), O.newton_schulz(G, steps)) <= 2e-3
 
 
+def test_newton_schulz_random_shapes_scales_and_step_counts(env):
+    """Forty seeded draws of (rows, cols, input scale, iteration count) through fast_newtonschulz against the oracle:
+    single rows and columns, ragged edges, both orientations, 128- and 256-tile buckets, inputs from 1e-3 to 50 times
+    N(0,1) (the normalisation removes the scale), 0 to 5 iterations; bound 2e-2 relative Frobenius error as stated for
+    five iterations."""
+    import random
+    O, mu = env["O"], env["mu"]
+    rng = random.Random(1234)
+    worst = 0.0
+    for trial in range(40):
+        rows = rng.choice([1, 7, 33, 64, 100, 128, 200, 256, 300, 384, 512, 640, 768, 896, 1024])
+        cols = rng.choice([1, 9, 47, 64, 96, 128, 250, 256, 384, 512, 700, 768, 1024, 1536])
+        steps = rng.choice([0, 1, 3, 5])
+        scale = rng.choice([1e-3, 1.0, 50.0])
+        print(f"random ns trial {trial}: {rows}x{cols} steps {steps} scale {scale}", flush=True)
+        G = torch.randn(rows, cols, generator=torch.Generator().manual_seed(trial)) * scale
+        err = rel_fro(mu.fast_newtonschulz(G.to(env["dev"]), steps), O.newton_schulz(G, steps))
+        worst = max(worst, err)
+        assert err <= NS_TOL, (rows, cols, steps, scale, err)
+    print(f"worst error over the random draws: {worst:.3e}", flush=True)
+
+
 def test_newton_schulz_config1(env):
     """Benchmark config 1: 896x4864 fp32 N(0,1) from seed 0, five bf16 iterations."""
     print("ns config 1", flush=True)
