@@ -58,9 +58,10 @@ extern "C" {
 #define MUON_HIP_CFG_256_PIPE 1      /* 256x256 tile, 8 waves, the same pipeline */
 #define MUON_HIP_CFG_256_PINGPONG 2  /* 256x256 tile, two groups of 4 waves alternating memory / MFMA phases */
 #define MUON_HIP_CFG_128_PINGPONG 3  /* 128x128 tile, the same eight-wave kernel, two workgroups per compute unit */
-#define MUON_HIP_CFG_256_PERSIST 4   /* a.X + B.X as a persistent kernel: a workgroup per compute unit walks 256x256 tiles,
-                                        the next tile's first loads land behind the epilogue; the other products and
-                                        launches of at most one round take MUON_HIP_CFG_256_PINGPONG */
+#define MUON_HIP_CFG_256_PERSIST 4   /* the ping-pong loop as a persistent kernel: a workgroup per compute unit walks 256x256 tiles,
+                                        the next tile's first loads land behind an epilogue that needs no LDS.  Taken by launches
+                                        of more than one round of tiles: a.X + B.X, and the symmetric products with reductions
+                                        of at most 2048; everything else runs MUON_HIP_CFG_256_PINGPONG */
 #define MUON_HIP_CFG_COUNT 5
 
 int muon_hip_version(void);

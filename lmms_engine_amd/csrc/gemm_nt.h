@@ -14,9 +14,10 @@ enum {
     GEMM_CFG_256_PIPE = 1,      // 256x256 tile, 8 waves, the same pipeline
     GEMM_CFG_256_PINGPONG = 2,  // 256x256 tile, 8 waves in two alternating groups, four stages of 32 columns
     GEMM_CFG_128_PINGPONG = 3,  // 128x128 tile, the same eight-wave kernel, two workgroups per compute unit
-    GEMM_CFG_256_PERSIST = 4,   // a.X + B.X: the ping-pong loop as a persistent kernel (a workgroup per compute unit walks
-                                // tiles, the next tile's first loads land behind the LDS-free epilogue); other products
-                                // and launches of at most one round run GEMM_CFG_256_PINGPONG
+    GEMM_CFG_256_PERSIST = 4,   // the ping-pong loop as a persistent kernel (a workgroup per compute unit walks tiles, the next
+                                // tile's first loads land behind an epilogue without LDS): a.X + B.X, and the symmetric
+                                // products with reductions up to 2048; launches of at most one round and the launches that
+                                // carry the parameter update run GEMM_CFG_256_PINGPONG
     GEMM_CFG_COUNT = 5
 };
 
