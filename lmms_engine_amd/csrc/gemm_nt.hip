@@ -1076,8 +1076,8 @@ __global__ void __launch_bounds__(512) gemm_nt_pp_tail_kernel(const GemmArgs g) 
     }
 }
 
-// ---- kernel 3: a.X + B.X as a persistent kernel ------------------------------------------------
-// The epilogue of EPI_BX needs no LDS (epilogue_nn_reg), so nothing stands between the k loops of two tiles: one
+// ---- kernel 3: the ping-pong loop as a persistent kernel ----------------------------------------
+// With an epilogue that needs no LDS (epilogue_nn_reg, epilogue_sym_reg) nothing stands between the k loops of two tiles: one
 // workgroup per compute unit walks tiles, the last three memory phases of a tile issue the first three k-tiles of the
 // workgroup's NEXT tile into the stages the current one has finished with, and they land while the waves drain their
 // accumulators.  What a one-tile workgroup pays around its k loop on top of the epilogue - the cold first loads (2 to
