@@ -37,9 +37,11 @@ logger = logging.getLogger(__name__)
 NS_COEFFS = (3.4445, -4.7750, 2.0315)  # muon_utils.py:137
 
 # Cap of the Newton-Schulz workspace one grouped launch may use; buckets that need more are cut into chunks.
-# Measured on the Qwen3-8B-shaped set: 1 / 2 / 4 / 8 / 24 GiB give 382 / 373 / 375 / 380 / 384 ms per step (chunks of
-# a few large matrices keep the operands of one launch closer to the memory-side cache), so the default is 2 GiB.
-DEFAULT_WORKSPACE_LIMIT = 2 << 30
+# Measured on the Qwen3-8B-shaped set: 2 / 3.2 / 4.2 / 5 / 6.5 / 8.5 GiB give 357.9 / 353.2 / 352.0 / 351.4 / 351.6 /
+# 352.2 ms per step: up to about 4 GiB larger chunks land the triangular tile counts of X.Xt on whole rounds of the compute
+# units (15 matrices 4096x12288 = 2040 tiles = 7.97 rounds, where 7 gave 3.72), past that a.X + B.X loses what chunks of a few
+# large matrices gain from the memory-side cache.  4 GiB is the smallest cap within 0.2 % of the best.
+DEFAULT_WORKSPACE_LIMIT = 4 << 30
 
 _noted_semantics = False
 
