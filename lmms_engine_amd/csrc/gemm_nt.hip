@@ -1221,99 +1221,99 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_kernel(const GemmArgs g) {
         // One tile, k loop and epilogue, for the waves whose skip mask in a diagonal tile is `mask_c` (pp_tile): a copy of
         // its own per mask, each with its own accumulators from the first MFMA to the last store.
         auto run_tile = [&](auto mask_c) {
-        f32x4 acc[FM][FN];  // defined by the MFMAs of the tile's first k-tile, which add to zero
+            f32x4 acc[FM][FN];  // defined by the MFMAs of the tile's first k-tile, which add to zero
 
-        // NEXT: the memory phase issues k-tile kt+3-nk of the next tile instead of k-tile kt+3 of this one.
-        // NOWAIT: the first two phases of a tile wait for no load: its k-tiles 0, 1 and 2 are in LDS when it starts
-        // (a count would make them wait for the stores of the epilogue before).
-        constexpr unsigned MASK = decltype(mask_c)::value;  // fragments a wave skips in a diagonal tile
-        auto body = [&](int kt, auto stage_c, auto next_c, auto nowait_c, auto first_c) {
-            constexpr int SIDX = decltype(stage_c)::value;
-            constexpr bool NEXT = decltype(next_c)::value;
-            constexpr bool NOWAIT = decltype(nowait_c)::value;
-            constexpr bool FIRST = decltype(first_c)::value;
-            auto kept = [](int i, int j) { return !((MASK >> (i * FN + j)) & 1); };
-            bf16x8 fa[FM], fb[FN];
-#pragma unroll
-            for (int i = 0; i < FM; ++i) {
-                bool used = false;
-#pragma unroll
-                for (int j = 0; j < FN; ++j) used |= kept(i, j);
-                if (used) fa[i] = *(const bf16x8*)(ra[SIDX >> 1] + (SIDX & 1) * STAGE + i * 16 * ROWB);
-            }
-#pragma unroll
-            for (int j = 0; j < FN; ++j) {
-                bool used = false;
-#pragma unroll
-                for (int i = 0; i < FM; ++i) used |= kept(i, j);
-                if (!used) continue;
-                if (QT) fb[j] = lds_read_qt(rb[SIDX >> 1][j & 1] + (SIDX & 1) * STAGE + (j >> 1) * 2048);
-                else fb[j] = *(const bf16x8*)(rb[SIDX >> 1][0] + (SIDX & 1) * STAGE + j * 16 * ROWB);
-            }
-            if constexpr (NEXT) issue_tile(Pn, Qn, kt + 3 - nk);
-            else issue_tile(Pb, Qb, kt + 3);
-            WAIT_LGKM0();
-            if constexpr (!NOWAIT) WAIT_VM(2 * NLD);  // own loads of k-tile kt+1 have landed
-            __builtin_amdgcn_sched_barrier(0);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int j = 0; j < FN; ++j)
-#pragma unroll
-                for (int ii = 0; ii < FM; ++ii) {
-                    const int i = (j & 1) ? FM - 1 - ii : ii;  // back and forth: consecutive MFMAs share an operand
-                    const f32x4 c = FIRST ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[i][j];
-                    if (QT) acc[i][j] = mfma16(fb[j], fa[i], c);
-                    else if (kept(i, j)) acc[i][j] = mfma16(fa[i], fb[j], c);
+            // NEXT: the memory phase issues k-tile kt+3-nk of the next tile instead of k-tile kt+3 of this one.
+            // NOWAIT: the first two phases of a tile wait for no load: its k-tiles 0, 1 and 2 are in LDS when it starts
+            // (a count would make them wait for the stores of the epilogue before).
+            constexpr unsigned MASK = decltype(mask_c)::value;  // fragments a wave skips in a diagonal tile
+            auto body = [&](int kt, auto stage_c, auto next_c, auto nowait_c, auto first_c) {
+                constexpr int SIDX = decltype(stage_c)::value;
+                constexpr bool NEXT = decltype(next_c)::value;
+                constexpr bool NOWAIT = decltype(nowait_c)::value;
+                constexpr bool FIRST = decltype(first_c)::value;
+                auto kept = [](int i, int j) { return !((MASK >> (i * FN + j)) & 1); };
+                bf16x8 fa[FM], fb[FN];
+    #pragma unroll
+                for (int i = 0; i < FM; ++i) {
+                    bool used = false;
+    #pragma unroll
+                    for (int j = 0; j < FN; ++j) used |= kept(i, j);
+                    if (used) fa[i] = *(const bf16x8*)(ra[SIDX >> 1] + (SIDX & 1) * STAGE + i * 16 * ROWB);
                 }
-            __builtin_amdgcn_sched_barrier(0);
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_s_barrier();
-            asm volatile("" ::: "memory");
-            __builtin_amdgcn_sched_barrier(0);
-        };
-        using I0 = std::integral_constant<int, 0>;
-        using I1 = std::integral_constant<int, 1>;
-        using I2 = std::integral_constant<int, 2>;
-        using I3 = std::integral_constant<int, 3>;
-        using No = std::false_type;
-        using Yes = std::true_type;
-        body(0, I0{}, No{}, Yes{}, Yes{});
-        body(1, I1{}, No{}, Yes{}, No{});
-        body(2, I2{}, No{}, No{}, No{});
-        body(3, I3{}, No{}, No{}, No{});
-        for (int kt = 4; kt < nk - 4; kt += 4) {
-            body(kt, I0{}, No{}, No{}, No{});
-            body(kt + 1, I1{}, No{}, No{}, No{});
-            body(kt + 2, I2{}, No{}, No{}, No{});
-            body(kt + 3, I3{}, No{}, No{}, No{});
-        }
-        body(nk - 4, I0{}, No{}, No{}, No{});
-        body(nk - 3, I1{}, Yes{}, No{}, No{});
-        body(nk - 2, I2{}, Yes{}, No{}, No{});
-        body(nk - 1, I3{}, Yes{}, No{}, No{});
-        if (!grp) __builtin_amdgcn_s_barrier();  // the two groups leave the k loop together
-        MUON_TRACE_STAMP_AT(g, pid_cur, 2);
+    #pragma unroll
+                for (int j = 0; j < FN; ++j) {
+                    bool used = false;
+    #pragma unroll
+                    for (int i = 0; i < FM; ++i) used |= kept(i, j);
+                    if (!used) continue;
+                    if (QT) fb[j] = lds_read_qt(rb[SIDX >> 1][j & 1] + (SIDX & 1) * STAGE + (j >> 1) * 2048);
+                    else fb[j] = *(const bf16x8*)(rb[SIDX >> 1][0] + (SIDX & 1) * STAGE + j * 16 * ROWB);
+                }
+                if constexpr (NEXT) issue_tile(Pn, Qn, kt + 3 - nk);
+                else issue_tile(Pb, Qb, kt + 3);
+                WAIT_LGKM0();
+                if constexpr (!NOWAIT) WAIT_VM(2 * NLD);  // own loads of k-tile kt+1 have landed
+                __builtin_amdgcn_sched_barrier(0);
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for (int j = 0; j < FN; ++j)
+    #pragma unroll
+                    for (int ii = 0; ii < FM; ++ii) {
+                        const int i = (j & 1) ? FM - 1 - ii : ii;  // back and forth: consecutive MFMAs share an operand
+                        const f32x4 c = FIRST ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[i][j];
+                        if (QT) acc[i][j] = mfma16(fb[j], fa[i], c);
+                        else if (kept(i, j)) acc[i][j] = mfma16(fa[i], fb[j], c);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            using I0 = std::integral_constant<int, 0>;
+            using I1 = std::integral_constant<int, 1>;
+            using I2 = std::integral_constant<int, 2>;
+            using I3 = std::integral_constant<int, 3>;
+            using No = std::false_type;
+            using Yes = std::true_type;
+            body(0, I0{}, No{}, Yes{}, Yes{});
+            body(1, I1{}, No{}, Yes{}, No{});
+            body(2, I2{}, No{}, No{}, No{});
+            body(3, I3{}, No{}, No{}, No{});
+            for (int kt = 4; kt < nk - 4; kt += 4) {
+                body(kt, I0{}, No{}, No{}, No{});
+                body(kt + 1, I1{}, No{}, No{}, No{});
+                body(kt + 2, I2{}, No{}, No{}, No{});
+                body(kt + 3, I3{}, No{}, No{}, No{});
+            }
+            body(nk - 4, I0{}, No{}, No{}, No{});
+            body(nk - 3, I1{}, Yes{}, No{}, No{});
+            body(nk - 2, I2{}, Yes{}, No{}, No{});
+            body(nk - 1, I3{}, Yes{}, No{}, No{});
+            if (!grp) __builtin_amdgcn_s_barrier();  // the two groups leave the k loop together
+            MUON_TRACE_STAMP_AT(g, pid_cur, 2);
 
-        // Every wave drains its accumulators on its own.  One lane asks for the id of the tile after the next (an
-        // increment with wrap-around at 2^32 - 1: a plain atomicAdd of a uniform value is turned into a wave-wide
-        // reduction by the compiler, which then waits for the answer on the spot); the answer is needed at the end.
-        if (has_next && tid == 0) fetched = atomicInc(&g_ppx[g.ppx_slot].next[xcd][0], 0xffffffffu);
-        if constexpr (QT) {
-            epilogue_nn_reg<BM, BN, WGM, WGN>(g, tc, acc);
-        } else {
-            epilogue_sym_reg<BM, BN, WGM, WGN, EPI, MASK>(g, tc, acc);
-            // What says that this wave's share of the next tile's first k-tiles has landed: B.X and b.A + c.A.A consume
-            // loads that were issued after them (the queue returns in order).  X.Xt loads nothing, and in a diagonal
-            // tile a wave may have nothing to finish at all: there the count is explicit (48 stores went out after the
-            // loads off the diagonal, an unknown number on it).
-            asm volatile("" ::: "memory");
-            if (diag) WAIT_VM(0);
-            else if (EPI == EPI_SYRK) WAIT_VM(FM * FN / 2 * 3);
-            asm volatile("" ::: "memory");
-        }
+            // Every wave drains its accumulators on its own.  One lane asks for the id of the tile after the next (an
+            // increment with wrap-around at 2^32 - 1: a plain atomicAdd of a uniform value is turned into a wave-wide
+            // reduction by the compiler, which then waits for the answer on the spot); the answer is needed at the end.
+            if (has_next && tid == 0) fetched = atomicInc(&g_ppx[g.ppx_slot].next[xcd][0], 0xffffffffu);
+            if constexpr (QT) {
+                epilogue_nn_reg<BM, BN, WGM, WGN>(g, tc, acc);
+            } else {
+                epilogue_sym_reg<BM, BN, WGM, WGN, EPI, MASK>(g, tc, acc);
+                // What says that this wave's share of the next tile's first k-tiles has landed: B.X and b.A + c.A.A consume
+                // loads that were issued after them (the queue returns in order).  X.Xt loads nothing, and in a diagonal
+                // tile a wave may have nothing to finish at all: there the count is explicit (48 stores went out after the
+                // loads off the diagonal, an unknown number on it).
+                asm volatile("" ::: "memory");
+                if (diag) WAIT_VM(0);
+                else if (EPI == EPI_SYRK) WAIT_VM(FM * FN / 2 * 3);
+                asm volatile("" ::: "memory");
+            }
         };  // run_tile
         if (!diag) {
             run_tile(std::integral_constant<unsigned, 0>{});
