@@ -561,18 +561,18 @@ __device__ __forceinline__ void epilogue_sym_reg(const GemmArgs& g, const TileCo
                 (wm * WTM + 4 * row + (lane & 3)) * BLK_COLS + ((lane >> 2) & 3) * 4;
     const unsigned sel = (lane & 1) ? 0x03020706u : 0x05040100u;
     const bool upper = (lane & 2) != 0;
-    // SYMPOLY: the b.A pieces of all but the last row of pairs are fetched up front, those of the last row once the
-    // first row is finished and its registers are free
+    // SYMPOLY: the b.A pieces of EV_AHEAD rows of pairs are in flight at a time; those of row t + EV_AHEAD are fetched
+    // when row t starts (all of them at once do not fit beside the accumulators in the persistent kernel)
     bf16x8 ev[EPI == EPI_SYMPOLY ? FM / 2 : 1][EPI == EPI_SYMPOLY ? FN : 1];
     const bf16_t* Et = g.Et + tc.bidx * g.strideEt + panel_offset(n0, g.cbEt) + ct_off;
-    constexpr int EV_LATE = FM / 2 > 2 ? FM / 2 - 1 : FM / 2;  // first row of pairs that is fetched late
+    constexpr int EV_AHEAD = 2 < FM / 2 ? 2 : FM / 2;  // measured: 3 no faster, 4 spills an accumulator fragment
     auto load_ev = [&](int t) {
 #pragma unroll
         for (int j = 0; j < FN; ++j) ev[t][j] = *(const bf16x8*)(Et + j * 16 * BLK_COLS + (long)t * BLK_ELEMS);
     };
     if constexpr (EPI == EPI_SYMPOLY) {
 #pragma unroll
-        for (int t = 0; t < EV_LATE; ++t) load_ev(t);
+        for (int t = 0; t < EV_AHEAD; ++t) load_ev(t);
     }
     auto rounded = [&](float v) {
         v = rbf(v);
@@ -582,7 +582,7 @@ __device__ __forceinline__ void epilogue_sym_reg(const GemmArgs& g, const TileCo
 #pragma unroll
     for (int t = 0; t < FM / 2; ++t) {
         if constexpr (EPI == EPI_SYMPOLY) {
-            if (t == 1 && EV_LATE < FM / 2) load_ev(EV_LATE);
+            if (t + EV_AHEAD < FM / 2) load_ev(t + EV_AHEAD);
         }
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
