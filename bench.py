@@ -336,6 +336,8 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the workload's own)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--hip-graph", action="store_true",
+                    help="record one step into a HIP graph after the warm-up and time its replays (no per-kernel timing)")
     ap.add_argument("--workspace-limit-gib", type=float, default=0.0,
                     help="cap of the Newton-Schulz workspace (0 = the optimizer's default); smaller caps mean more, "
                          "smaller grouped launches")
@@ -403,6 +405,14 @@ def main():
     for _ in range(args.warmup):
         opt.step()
     torch.cuda.synchronize()
+    step_fn = opt.step
+    if args.hip_graph:
+        args.no_kernel_timing = True  # events around every launch do not record into a graph
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            opt.step()
+        step_fn = graph.replay
+        torch.cuda.synchronize()
     if not args.no_kernel_timing:
         _abi.timing_enable(True)
     # one event per step boundary on the stream the kernels run on: per-step times for the median and the minimum
@@ -410,7 +420,7 @@ def main():
     t0 = time.perf_counter()
     marks[0].record()
     for i in range(args.steps):
-        opt.step()
+        step_fn()
         marks[i + 1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
@@ -485,7 +495,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.workload} 2-D parameter set, {layers} layers, {len(shapes)} matrices, "
                                f"{w['pdtype']} params/grads, fp32 momentum, full Muon step",
-                   "elements": elements, "ns_steps": HP["ns_steps"], "grouped_buckets": len(set(shapes))},
+                   "elements": elements, "ns_steps": HP["ns_steps"], "grouped_buckets": len(set(shapes)),
+                   "launch": "replays of one step recorded into a HIP graph" if args.hip_graph else "eager"},
         "ns_flop_per_step_algorithmic": flops_step,
         "pct_bf16_mfma_peak_whole_step": 100.0 * flops_step / (ms_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "ns_tflops_gemm_kernels_only": (flops_step / (gemm_ms * 1e-3) / 1e12) if gemm_ms else None,

@@ -76,9 +76,20 @@ def _workspace(nbytes: int, device) -> Tensor:
     return torch.empty(nbytes, dtype=torch.uint8, device=device)
 
 
-def _pointer_table(tensors, device) -> Tensor:
-    host = torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64, pin_memory=True)
-    return host.to(device, non_blocking=True)
+def _pointer_table(tensors, device, cache=None, key=None) -> Tensor:
+    """Device table of the tensors' base pointers.  With a cache, a table whose pointers have not changed since the last
+    call under `key` is handed back as it is: no host allocation and no copy, which is what lets a step over static
+    tensors be recorded into a HIP graph (and saves the copy otherwise)."""
+    ptrs = tuple(t.data_ptr() for t in tensors)
+    if cache is not None:
+        hit = cache.get(key)
+        if hit is not None and hit[0] == ptrs and hit[1].device == device:
+            return hit[1]
+    host = torch.tensor(ptrs, dtype=torch.int64, pin_memory=True)
+    table = host.to(device, non_blocking=True)
+    if cache is not None:
+        cache[key] = (ptrs, table)
+    return table
 
 
 def scale_factor(rows: int, cols: int, rms_scale: bool) -> float:
@@ -283,7 +294,7 @@ def _pick_chunk(n: int, cap: int, rows: int, cols: int) -> int:
     return best
 
 
-def _muon_bucket_step(params, grads, moms, group, ns_steps, nesterov, write_back_grad, ws_holder, ws_limit):
+def _muon_bucket_step(params, grads, moms, group, ns_steps, nesterov, write_back_grad, ws_holder, ws_limit, tables=None):
     """All stages of the Muon step for same-shape, same-dtype parameters on one device."""
     p0 = params[0]
     rows, cols = p0.shape
@@ -305,7 +316,8 @@ def _muon_bucket_step(params, grads, moms, group, ns_steps, nesterov, write_back
             if ws is None or ws.numel() < need:
                 ws_holder[dev] = None
                 ws = ws_holder[dev] = _workspace(need, dev)
-            table = _pointer_table(params[lo:hi] + grads[lo:hi] + moms[lo:hi], dev)
+            table = _pointer_table(params[lo:hi] + grads[lo:hi] + moms[lo:hi], dev, tables,
+                                   (dev, rows, cols, p0.dtype, grads[0].dtype, moms[0].dtype, lo))
             base = table.data_ptr()
             _abi.check(
                 lib.muon_hip_step_grouped(
@@ -401,6 +413,7 @@ class Muon(torch.optim.Optimizer):
         self.workspace_limit_bytes = int(workspace_limit_bytes)
         self.keep_workspace = bool(keep_workspace)
         self._workspaces = {}
+        self._pointer_tables = {}  # per bucket chunk: (pointers, device table) of the last step
         if not reference_bug_compat and not is_deepspeed_enabled:
             _note_keyword_semantics()
         for group in param_groups:
@@ -554,7 +567,7 @@ class Muon(torch.optim.Optimizer):
                 for items in buckets.values():
                     ps, gs, ms = (list(t) for t in zip(*items))
                     _muon_bucket_step(ps, gs, ms, group, ns_steps, nesterov, self.write_back_grad, self._workspaces,
-                                      self.workspace_limit_bytes)
+                                      self.workspace_limit_bytes, self._pointer_tables)
             else:
                 self._adam_group_step(group)
 

@@ -766,6 +766,42 @@ def test_module_substitution_factory_groups_and_checkpoint_round_trip(env, tmp_p
         assert torch.equal(ps[k].detach(), ps2[k].detach()), k
 
 
+def test_muon_step_replays_from_a_hip_graph(env):
+    """A step over static tensors records into a HIP graph (the pointer tables of the last step are reused, so nothing is
+    allocated or copied while recording) and every replay equals the eager step of a twin optimizer bit for bit: four
+    replays, each followed by the twin's eager step and a synchronisation.  The set holds buckets that run the persistent
+    kernels (their tile counters are taken at record time and must come back to zero after every replay), a transposed
+    bucket and a 128-tile one."""
+    dev, mu = env["dev"], env["mu"]
+    shapes = [(768, 2048)] * 60 + [(1024, 512)] * 4 + [(384, 640)] * 3
+
+    def make():
+        g = torch.Generator().manual_seed(5)
+        ps = [torch.nn.Parameter((torch.randn(r, c, generator=g) * 0.02).bfloat16().to(dev)) for r, c in shapes]
+        for p in ps:
+            p.grad = (torch.randn(p.shape, generator=g) * 0.01).bfloat16().to(dev)
+        opt = mu.Muon([dict(params=ps, use_muon=True, lr=0.02, momentum=0.95, weight_decay=0.01, rms_scale=False)],
+                      momentum_dtype=torch.float32)
+        return ps, opt
+
+    (pa, oa), (pb, ob) = make(), make()
+    for _ in range(2):  # state, workspace and pointer tables exist after the first steps
+        oa.step()
+        ob.step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        oa.step()
+    for rep in range(4):
+        print(f"graph replay {rep}", flush=True)
+        graph.replay()
+        ob.step()
+        torch.cuda.synchronize()
+        for i, (p, q) in enumerate(zip(pa, pb)):
+            assert torch.equal(p, q), (rep, i, shapes[i])
+            assert torch.equal(oa.state[p]["momentum_buffer"], ob.state[q]["momentum_buffer"]), (rep, i)
+
+
 def test_reference_bug_compat_and_rms_scale(env):
     """The reference's single-device call site runs range(True) = 1 NS iteration; the flag reproduces it."""
     mu, O = env["mu"], env["O"]
