@@ -317,7 +317,7 @@ def _muon_bucket_step(params, grads, moms, group, ns_steps, nesterov, write_back
                 ws_holder[dev] = None
                 ws = ws_holder[dev] = _workspace(need, dev)
             table = _pointer_table(params[lo:hi] + grads[lo:hi] + moms[lo:hi], dev, tables,
-                                   (dev, rows, cols, p0.dtype, grads[0].dtype, moms[0].dtype, lo))
+                                   (id(group), dev, rows, cols, p0.dtype, grads[0].dtype, moms[0].dtype, lo))
             base = table.data_ptr()
             _abi.check(
                 lib.muon_hip_step_grouped(
