@@ -1364,15 +1364,25 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_kernel(const GemmArgs g) {
 
 std::atomic<unsigned> g_ppx_sequence{0};  // launches take the counter slots in turn
 
+// Dynamic LDS beyond 64 KB has to be allowed per kernel, and the attribute belongs to the device that is current when
+// it is set: once per (kernel instantiation, device), remembered as one bit per device in the instantiation's mask.
+hipError_t allow_dynamic_lds(const void* kern, int bytes, std::atomic<unsigned long long>& done) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return e;
+    done.fetch_or(bit, std::memory_order_release);
+    return hipSuccess;
+}
+
 template <int EPI>
 hipError_t launch_ppx(GemmArgs g, int nblocks, hipStream_t stream) {
     constexpr int smem = 4 * (256 + 256) * 64 + 64;
-    static std::atomic<bool> configured{false};  // per instantiation
-    if (!configured.load(std::memory_order_acquire)) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_nt_ppx_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        configured.store(true, std::memory_order_release);
-    }
+    static std::atomic<unsigned long long> configured{0};  // per instantiation
+    if (hipError_t e = allow_dynamic_lds((const void*)gemm_nt_ppx_kernel<EPI>, smem, configured); e != hipSuccess) return e;
     g.ppx_slot = (int)(g_ppx_sequence.fetch_add(1, std::memory_order_relaxed) % PPX_SLOTS);
     const int grid = nblocks < GEMM_CU_COUNT ? nblocks : GEMM_CU_COUNT;
     hipLaunchKernelGGL(gemm_nt_ppx_kernel<EPI>, dim3(grid), dim3(512), smem, stream, g);
@@ -1384,15 +1394,11 @@ hipError_t launch_one(const GemmArgs& g, int nblocks, hipStream_t stream) {
     constexpr int stages = 2 * (BM + BN) * ROW_BYTES;
     constexpr int epi = epi_is_bx(EPI) ? epilogue_nn_bytes<BM, BN>() : epilogue_bytes<BM, BN>();
     constexpr int smem = stages > epi ? stages : epi;
-    static std::atomic<bool> configured{false};  // per instantiation; setting the attribute twice is harmless
+    static std::atomic<unsigned long long> configured{0};  // per instantiation; setting the attribute twice is harmless
     void (*kern)(const GemmArgs);
     if constexpr (FEED == 1) kern = gemm_nt_pp_kernel<BM, BN, WGM, WGN, EPI>;
     else kern = gemm_nt_pipe_kernel<BM, BN, WGM, WGN, EPI>;
-    if (!configured.load(std::memory_order_acquire)) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        configured.store(true, std::memory_order_release);
-    }
+    if (hipError_t e = allow_dynamic_lds((const void*)kern, smem, configured); e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(nblocks), dim3(WGM * WGN * 64), smem, stream, g);
     return hipGetLastError();
 }
@@ -1426,13 +1432,9 @@ hipError_t launch_pp_tail(GemmArgs g, int nblocks, int rest, hipStream_t stream)
     constexpr int stages = 2 * (256 + 256) * ROW_BYTES;
     constexpr int epi = epi_is_bx(EPI) ? epilogue_nn_bytes<256, 256>() : epilogue_bytes<256, 256>();
     constexpr int smem = stages > epi ? stages : epi;  // the 128-tiles need less of both
-    static std::atomic<bool> configured{false};
+    static std::atomic<unsigned long long> configured{0};
     auto kern = gemm_nt_pp_tail_kernel<EPI>;
-    if (!configured.load(std::memory_order_acquire)) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        configured.store(true, std::memory_order_release);
-    }
+    if (hipError_t e = allow_dynamic_lds((const void*)kern, smem, configured); e != hipSuccess) return e;
     g.big_blocks = nblocks - rest;
     hipLaunchKernelGGL(kern, dim3(g.big_blocks + 4 * rest), dim3(512), smem, stream, g);
     return hipGetLastError();
