@@ -274,6 +274,7 @@ def operand_power(dev, M=4096, K=12288, nb=16, reps=10):
     Xo = torch.empty_like(X)
     A = torch.empty(nb * na, dtype=torch.bfloat16, device=dev)
     Bm = torch.empty_like(A)
+    ctr = torch.zeros(_abi.PPX_COUNTER_BYTES, dtype=torch.uint8, device=dev)  # tile counters of the persistent kernel
     res = {}
     for label in ("random", "constant"):
         if label == "random":
@@ -283,12 +284,12 @@ def operand_power(dev, M=4096, K=12288, nb=16, reps=10):
             X.fill_(1.0 / 128)
             A.fill_(1.0 / 64)
         calls = {
-            "syrk": (lambda: _abi.check(lib.muon_hip_syrk_bf16(X.data_ptr(), Bm.data_ptr(), M, K, nb, -1, _abi.stream_ptr(dev))),
+            "syrk": (lambda: _abi.check(lib.muon_hip_syrk_bf16(X.data_ptr(), Bm.data_ptr(), M, K, nb, -1, ctr.data_ptr(), _abi.stream_ptr(dev))),
                      float(M) * M * K * nb),
             "sympoly": (lambda: _abi.check(lib.muon_hip_sympoly_bf16(A.data_ptr(), Bm.data_ptr(), M, nb, -4.775, 2.0315, -1,
-                                                                     _abi.stream_ptr(dev))), float(M) ** 3 * nb),
+                                                                     ctr.data_ptr(), _abi.stream_ptr(dev))), float(M) ** 3 * nb),
             "bx_axpy": (lambda: _abi.check(lib.muon_hip_bx_axpy_bf16(A.data_ptr(), X.data_ptr(), Xo.data_ptr(), M, K, nb, 3.4445,
-                                                                     -1, _abi.stream_ptr(dev))), 2.0 * M * M * K * nb),
+                                                                     -1, ctr.data_ptr(), _abi.stream_ptr(dev))), 2.0 * M * M * K * nb),
         }
         res[label] = {}
         for name, (fn, flop) in calls.items():
@@ -300,25 +301,32 @@ def operand_power(dev, M=4096, K=12288, nb=16, reps=10):
 
 
 def mfma_probe(dev, iters=40000, reps=25):
-    """Loops of nothing but MFMAs (muon_hip_mfma_probe): both instruction shapes, operands with random mantissas
-    and constant operands.  The sustained rate is what the part's power management leaves of the 2.5 PFLOP/s."""
+    """Loops of nothing but MFMAs (muon_probe_mfma of libmuon_probe.so, a measurement library beside the product's):
+    both instruction shapes, operands with random mantissas and constant operands.  The sustained rate is what the
+    part's power management leaves of the 2.5 PFLOP/s."""
     import ctypes
 
     import torch
 
     from lmms_engine_amd import _abi
+    from lmms_engine_amd.build import PROBE_LIB
 
-    lib = _abi.lib()
-    n = _abi.PROBE_OPERAND_BYTES // 2
-    sink = torch.empty(_abi.PROBE_SINK_FLOATS, dtype=torch.float32, device=dev)
+    lib = ctypes.CDLL(PROBE_LIB)
+    lib.muon_probe_mfma.restype = ctypes.c_int
+    lib.muon_probe_mfma.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                    ctypes.POINTER(ctypes.c_double), ctypes.c_void_p]
+    n = 256 * 12 * 512 * 16 // 2
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
     res = {}
     for label in ("random", "constant"):
         ops = (torch.randn(n, device=dev) * 0.02).bfloat16() if label == "random" else torch.full((n,), 0.0078125, dtype=torch.bfloat16, device=dev)
         res[label] = {}
         for shape, name in ((0, "v_mfma_f32_32x32x16_bf16"), (1, "v_mfma_f32_16x16x32_bf16")):
             flop = ctypes.c_double()
-            fn = lambda: _abi.check(lib.muon_hip_mfma_probe(ops.data_ptr(), sink.data_ptr(), shape, iters, ctypes.byref(flop),
-                                                            _abi.stream_ptr(dev)))
+            def fn():
+                rc = lib.muon_probe_mfma(ops.data_ptr(), sink.data_ptr(), shape, iters, ctypes.byref(flop), _abi.stream_ptr(dev))
+                assert rc == 0, f"muon_probe_mfma failed ({rc})"
+
             # about half a second of back-to-back launches behind a warm-up of the same kind: the clock follows
             # the power drawn over tens of milliseconds
             ms = _event_ms(fn, reps, torch, warm=8)
@@ -414,7 +422,13 @@ def main():
         step_fn = graph.replay
         torch.cuda.synchronize()
     if not args.no_kernel_timing:
-        _abi.timing_enable(True)
+        # Event pairs for every launch of the timed region exist before it starts (one more warm-up step counts the
+        # launches of a step), so that a timed launch costs two event records and nothing else.
+        _abi.timing_enable(True, reserve=1 << 16)
+        step_fn()
+        torch.cuda.synchronize()
+        per_step = sum(cnt for _, cnt in _abi.timing_read().values())
+        _abi.timing_enable(True, reserve=per_step * args.steps + 64)
     # one event per step boundary on the stream the kernels run on: per-step times for the median and the minimum
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
@@ -430,7 +444,9 @@ def main():
     kern = {}
     if not args.no_kernel_timing:
         kern = _abi.timing_read()
+        untimed = _abi.lib().muon_hip_timing_untimed()
         _abi.timing_enable(False)
+        assert untimed == 0, f"{untimed} launches ran without events: the pool was too small"
 
     # per-kernel algorithmic work of one step
     syrk_f = sum(HP["ns_steps"] * float(min(s)) ** 2 * max(s) for s in shapes)

@@ -21,6 +21,13 @@
  *  - The Newton-Schulz operands live, in a blocked layout (below), in a caller-allocated workspace of
  *    muon_hip_workspace_bytes() bytes, 256-byte aligned, which the entry points partition
  *    identically; its contents between calls are private to the library.
+ *  - Concurrency.  The library keeps no device state of its own (the one exception is
+ *    muon_hip_grad_norms_static, which says so).  Everything a call shares between its kernels lives in
+ *    the caller's workspace, the tile counters of the persistent GEMM kernels included (the
+ *    normalisation stage clears them, every persistent launch leaves them zero).  Calls that use
+ *    different workspaces may run at the same time on different streams, also a replayed HIP graph beside
+ *    eager calls; calls that share a workspace (or a counter buffer of the single-GEMM entry points) must
+ *    be ordered on one stream, as for any other buffer both would write.
  */
 #ifndef MUON_HIP_H
 #define MUON_HIP_H
@@ -145,20 +152,25 @@ int muon_hip_unpack_bf16(const void* src, int rows_p, int cols_p, void* dst, lon
                          int batch, void* stream);
 
 /* The three products on explicit blocked buffers already padded to whole tiles (Mp, Kp multiples
- * of the configuration's tile edge). */
+ * of the configuration's tile edge).  `counters` is either null or MUON_HIP_PPX_COUNTER_BYTES of device
+ * memory, 64-byte aligned and zero before its first use: the tile counters that the persistent kernel
+ * (MUON_HIP_CFG_256_PERSIST) needs.  Every launch leaves the buffer zero again; launches that share it must
+ * be ordered on one stream.  With a null pointer the one-tile kernels run instead (same results bit for bit). */
+#define MUON_HIP_PPX_COUNTER_BYTES 576
 
 /* A (Mp x Mp) = bf16(X Xt) for X (Mp x Kp): matmul_transpose_assign + mmt_kernel,
  * muon_utils.py:95-119 and :28-92.  Upper tiles computed, mirrored below the diagonal. */
-int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* stream);
+int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* counters, void* stream);
 
 /* B = bf16(bf16(b*A) + bf16(c*bf16(A A))) for symmetric A (Mp x Mp): muon_utils.py:150-151. */
-int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* stream);
+int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* counters,
+                          void* stream);
 
 /* X' = bf16(bf16(a*X) + bf16(B X)): muon_utils.py:152.  B (Mp x Mp) symmetric, X and Xout (Mp x Kp) distinct
  * buffers.  The reduction runs down the columns of X, which the kernel reads from LDS with gfx950's
  * transposing read, so no transposed copy of X exists anywhere. */
 int muon_hip_bx_axpy_bf16(const void* B, const void* X, void* Xout, int Mp, int Kp, int batch, double a, int cfg,
-                          void* stream);
+                          void* counters, void* stream);
 
 /* ---- AdamW fallback ------------------------------------------------------------------ */
 
@@ -227,21 +239,22 @@ int muon_hip_grad_norms_static(const void* const* g_ptrs, const long* numel, con
 int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
                         int dtype, const float* total_f32, int norm_dtype, double max_norm, void* stream);
 
+/* Shape of the current device as the launchers see it, read from the runtime once per device: compute units
+ * (a round of 256x256 tiles is one per compute unit) and XCDs (compute units / 32 on gfx950, whole XCDs per
+ * partition).  No counterpart in the reference.  Either pointer may be null. */
+int muon_hip_device_shape(int* compute_units, int* xcds);
+
 /* ---- per-kernel timing ----------------------------------------------------------------
  * No counterpart in the reference.  When enabled, every kernel launch is bracketed by a pair
  * of HIP events on its own stream; muon_hip_timing_read waits for them and returns the summed
- * duration and launch count of one kernel id since timing was enabled. */
+ * duration and launch count of one kernel id since timing was enabled.  The events come from a pool:
+ * muon_hip_timing_reserve(n), called while timing is off, makes sure n pairs exist (enabling creates
+ * 4096 if there are fewer), so that a timed launch creates nothing and takes no lock.  Launches beyond
+ * the pool run untimed; muon_hip_timing_untimed() counts them since timing was enabled. */
+int muon_hip_timing_reserve(long launches);
 int muon_hip_timing_enable(int on);
-
-/* A loop of nothing but MFMAs, for measuring what the matrix pipes sustain under the part's power management.
- * No counterpart in the reference.  shape 0: v_mfma_f32_32x32x16_bf16, shape 1: v_mfma_f32_16x16x32_bf16, on one
- * workgroup of 8 waves per compute unit with the register footprint of the GEMM kernels.  `operands` holds
- * MUON_HIP_PROBE_OPERAND_BYTES of bf16 values chosen by the caller (random, constant ...), `sink` receives
- * MUON_HIP_PROBE_SINK_FLOATS floats; *flop is the work of the launch.  Time it with events on `stream`. */
-#define MUON_HIP_PROBE_OPERAND_BYTES (256L * 12 * 512 * 16)
-#define MUON_HIP_PROBE_SINK_FLOATS (256L * 512)
-int muon_hip_mfma_probe(const void* operands, void* sink, int shape, int iters, double* flop, void* stream);
 int muon_hip_timing_read(int kernel_id, double* total_ms, long* launches);
+long muon_hip_timing_untimed(void);
 
 #ifdef __cplusplus
 }

@@ -22,7 +22,7 @@ KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "app
                 "grad_norm", "clip_scale", "bx_axpy_update"]
 MULTI_CHUNK = 16384  # MUON_HIP_MULTI_CHUNK
 STATIC_MAX_CHUNKS = 1 << 20  # MUON_HIP_STATIC_MAX_CHUNKS
-PROBE_OPERAND_BYTES, PROBE_SINK_FLOATS = 256 * 12 * 512 * 16, 256 * 512  # MUON_HIP_PROBE_*
+PPX_COUNTER_BYTES = 576  # MUON_HIP_PPX_COUNTER_BYTES
 
 # name -> (restype, argtypes); mirrors include/muon_hip.h one to one
 SIGNATURES = {
@@ -45,9 +45,10 @@ SIGNATURES = {
     "muon_hip_blocked_elems": (c_long, [c_int, c_int]),
     "muon_hip_pack_bf16": (c_int, [c_void_p, c_long, c_int, c_int, c_int, c_void_p, c_int, c_int, c_int, c_void_p]),
     "muon_hip_unpack_bf16": (c_int, [c_void_p, c_int, c_int, c_void_p, c_long, c_int, c_int, c_int, c_int, c_void_p]),
-    "muon_hip_syrk_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
-    "muon_hip_sympoly_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_double, c_double, c_int, c_void_p]),
-    "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_int, c_void_p]),
+    "muon_hip_syrk_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "muon_hip_sympoly_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_double, c_double, c_int, c_void_p, c_void_p]),
+    "muon_hip_bx_axpy_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_int, c_void_p,
+                                      c_void_p]),
     "muon_hip_adamw": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_double,
                                c_double, c_double, c_double, c_void_p]),
     "muon_hip_adam_update": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_double,
@@ -60,7 +61,9 @@ SIGNATURES = {
     "muon_hip_total_norm": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "muon_hip_clip_scale": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_int, c_double,
                                     c_void_p]),
-    "muon_hip_mfma_probe": (c_int, [c_void_p, c_void_p, c_int, c_int, POINTER(c_double), c_void_p]),
+    "muon_hip_device_shape": (c_int, [POINTER(c_int), POINTER(c_int)]),
+    "muon_hip_timing_reserve": (c_int, [c_long]),
+    "muon_hip_timing_untimed": (c_long, []),
     "muon_hip_timing_enable": (c_int, [c_int]),
     "muon_hip_timing_read": (c_int, [c_int, POINTER(c_double), POINTER(c_long)]),
 }
@@ -121,7 +124,19 @@ def workspace_bytes(rows: int, cols: int, batch: int) -> int:
     return n
 
 
-def timing_enable(on: bool) -> None:
+def device_shape():
+    """(compute units, XCDs) of the current device."""
+    cus, xcds = c_int(), c_int()
+    check(lib().muon_hip_device_shape(ctypes.byref(cus), ctypes.byref(xcds)), "device_shape")
+    return cus.value, xcds.value
+
+
+def timing_enable(on: bool, reserve: int = 0) -> None:
+    """Switch per-kernel event timing on or off; `reserve` event pairs are created first, so that none has to be
+    created while the clock runs (launches beyond the pool go untimed and are counted by muon_hip_timing_untimed)."""
+    if on and reserve:
+        check(lib().muon_hip_timing_enable(0), "timing_enable")
+        check(lib().muon_hip_timing_reserve(int(reserve)), "timing_reserve")
     check(lib().muon_hip_timing_enable(int(on)), "timing_enable")
 
 

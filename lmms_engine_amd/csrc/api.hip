@@ -2,16 +2,19 @@
 // partitioning, the grouped launch sequence of one Muon step, and per-kernel event timing.
 #include <stdarg.h>
 #include <stdio.h>
+#include <algorithm>
 #include <atomic>
 #include <mutex>
 #include <vector>
 
+// The library is built with hidden visibility; the entry points declared in the public header are what it exports.
+#pragma GCC visibility push(default)
 #include "../../include/muon_hip.h"
+#pragma GCC visibility pop
 #include "common.h"
 #include "elementwise.h"
 #include "gemm_nt.h"
 #include "multi_tensor.h"
-#include "probe.h"
 
 namespace {
 
@@ -32,45 +35,54 @@ int hip_fail(hipError_t e, const char* what) {
 }
 
 // ---- timing ------------------------------------------------------------------------
+// Event pairs come from a pool that muon_hip_timing_reserve fills ahead of the region to be measured, so that a timed
+// launch costs two hipEventRecord calls and one atomic increment: no event is created and no lock is taken while the
+// clock runs.  A launch that finds the pool empty goes untimed and is counted in g_untimed.
 struct EventPair {
     hipEvent_t start, stop;
+    int kid;
 };
-std::mutex g_tmu;
+std::mutex g_tmu;                    // guards the pool's growth and the read-out, never a launch
 std::atomic<bool> g_timing{false};
-std::vector<EventPair> g_events[MUON_HIP_K_COUNT];
-constexpr size_t kMaxEventsPerKernel = 1 << 16;
+// The pool grows in chunks that are never moved or freed, so a launch may index it while another thread adds a chunk.
+constexpr size_t kPoolChunk = 4096, kPoolChunks = 256, kMaxPool = kPoolChunk * kPoolChunks;
+EventPair* g_chunks[kPoolChunks] = {};
+std::atomic<size_t> g_pool_size{0};  // pairs that exist
+std::atomic<size_t> g_used{0};       // pairs handed out since timing was enabled
+std::atomic<long> g_untimed{0};
+inline EventPair& pool_at(size_t i) { return g_chunks[i / kPoolChunk][i % kPoolChunk]; }
 
-void clear_events() {
-    for (auto& v : g_events) {
-        for (auto& p : v) {
+int grow_pool(size_t want) {  // under g_tmu
+    if (want > kMaxPool) want = kMaxPool;
+    for (size_t i = g_pool_size.load(std::memory_order_relaxed); i < want; ++i) {
+        if (i % kPoolChunk == 0 && !g_chunks[i / kPoolChunk]) g_chunks[i / kPoolChunk] = new EventPair[kPoolChunk]();
+        EventPair& p = pool_at(i);
+        if (hipError_t e = hipEventCreate(&p.start); e != hipSuccess) return hip_fail(e, "hipEventCreate");
+        if (hipError_t e = hipEventCreate(&p.stop); e != hipSuccess) {
             (void)hipEventDestroy(p.start);
-            (void)hipEventDestroy(p.stop);
+            return hip_fail(e, "hipEventCreate");
         }
-        v.clear();
+        g_pool_size.store(i + 1, std::memory_order_release);
     }
+    return 0;
 }
 
 struct Timed {
-    int kid;
+    EventPair* ev;
     hipStream_t s;
-    EventPair ev;
-    bool on;
-    Timed(int k, hipStream_t st) : kid(k), s(st), on(false) {
+    Timed(int kid, hipStream_t st) : ev(nullptr), s(st) {
         if (!g_timing.load(std::memory_order_acquire)) return;
-        std::lock_guard<std::mutex> lk(g_tmu);
-        if (g_events[kid].size() >= kMaxEventsPerKernel) return;
-        if (hipEventCreate(&ev.start) != hipSuccess) return;
-        if (hipEventCreate(&ev.stop) != hipSuccess) {
-            (void)hipEventDestroy(ev.start);
+        const size_t i = g_used.fetch_add(1, std::memory_order_relaxed);
+        if (i >= g_pool_size.load(std::memory_order_acquire)) {
+            g_untimed.fetch_add(1, std::memory_order_relaxed);
             return;
         }
-        on = hipEventRecord(ev.start, s) == hipSuccess;
+        ev = &pool_at(i);
+        ev->kid = kid;
+        if (hipEventRecord(ev->start, s) != hipSuccess) ev->kid = -1;
     }
     ~Timed() {
-        if (!on) return;
-        (void)hipEventRecord(ev.stop, s);
-        std::lock_guard<std::mutex> lk(g_tmu);
-        g_events[kid].push_back(ev);
+        if (ev && ev->kid >= 0 && hipEventRecord(ev->stop, s) != hipSuccess) ev->kid = -1;
     }
 };
 
@@ -79,7 +91,7 @@ struct Plan {
     int rows, cols, batch, M, K, Mp, Kp, tile, cfg, nparts;
     bool transposed;
     long n, strideU, strideX, strideA;  // elements per matrix: U dense, the others blocked
-    size_t offX[2], offA, offB, offParts, offDenom, total;
+    size_t offX[2], offA, offB, offParts, offDenom, offPpx, total;
 };
 
 inline long round_up(long v, long m) { return (v + m - 1) / m * m; }
@@ -138,15 +150,22 @@ int make_plan(int rows, int cols, int batch, Plan& p) {
     p.offB = seg(ab);
     p.offParts = seg((size_t)batch * p.nparts * sizeof(float));
     p.offDenom = seg((size_t)batch * sizeof(float));
+    p.offPpx = seg(GEMM_PPX_COUNTER_BYTES);  // tile counters of the persistent kernels: cleared by the normalisation stage
     p.total = off;
     return 0;
 }
 
 inline bf16_t* wsp(void* ws, size_t off) { return (bf16_t*)((char*)ws + off); }
+inline unsigned* ws_ppx(void* ws, const Plan& p) { return (unsigned*)((char*)ws + p.offPpx); }
 
 int check_ws(const void* ws) {
     if (!ws) return fail(MUON_HIP_EINVAL, "workspace is null");
     if (((uintptr_t)ws) & 255) return fail(MUON_HIP_EINVAL, "workspace must be 256-byte aligned");
+    return 0;
+}
+
+int check_counters(const void* counters) {
+    if (((uintptr_t)counters) & 63) return fail(MUON_HIP_EINVAL, "the counter buffer must be 64-byte aligned");
     return 0;
 }
 
@@ -160,15 +179,8 @@ int check_gemm(int cfg, int Mp, int Kp, int batch, int& tile) {
     return 0;
 }
 
-#ifdef MUON_TILE_TRACE
-long* g_trace = nullptr;  // measurement builds only
-#define SET_TRACE(g) (g).trace = g_trace
-#else
-#define SET_TRACE(g) do { } while (0)
-#endif
-
 // The three products on blocked buffers; matrix b of a batch starts at b * blocked_elems(rows, cols).
-int do_syrk(int cfg, const bf16_t* X, bf16_t* A, int Mp, int Kp, int batch, hipStream_t s) {
+int do_syrk(int cfg, const bf16_t* X, bf16_t* A, int Mp, int Kp, int batch, unsigned* ppx, hipStream_t s) {
     GemmArgs g = {};
     const int tile = gemm_cfg_tile(cfg), T = Mp / tile;
     g.P = g.Q = X;
@@ -180,13 +192,13 @@ int do_syrk(int cfg, const bf16_t* X, bf16_t* A, int Mp, int Kp, int batch, hipS
     g.C = g.Ct = A;
     g.strideC = g.strideCt = blocked_elems(Mp, Mp);
     g.cbC = g.cbCt = Mp / BLK_COLS;
-    SET_TRACE(g);
+    g.ppx = ppx;
     Timed t(MUON_HIP_K_SYRK, s);
     hipError_t e = launch_gemm_nt(cfg, EPI_SYRK, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "syrk launch");
 }
 
-int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b, double c, hipStream_t s) {
+int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b, double c, unsigned* ppx, hipStream_t s) {
     GemmArgs g = {};
     const int tile = gemm_cfg_tile(cfg), T = Mp / tile;
     g.P = g.Q = A;
@@ -203,7 +215,7 @@ int do_sympoly(int cfg, const bf16_t* A, bf16_t* B, int Mp, int batch, double b,
     g.cbEt = Mp / BLK_COLS;
     g.s0 = (float)b;
     g.s1 = (float)c;
-    SET_TRACE(g);
+    g.ppx = ppx;
     Timed t(MUON_HIP_K_SYMPOLY, s);
     hipError_t e = launch_gemm_nt(cfg, EPI_SYMPOLY, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "sympoly launch");
@@ -216,8 +228,8 @@ struct FoldUpdate {
     double scale, lr, weight_decay;
 };
 
-int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int Kp, int batch, double a, hipStream_t s,
-          const FoldUpdate* fold = nullptr) {
+int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int Kp, int batch, double a, unsigned* ppx,
+          hipStream_t s, const FoldUpdate* fold = nullptr) {
     GemmArgs g = {};
     const int tile = gemm_cfg_tile(cfg);
     g.P = B;
@@ -246,7 +258,7 @@ int do_bx(int cfg, const bf16_t* B, const bf16_t* X, bf16_t* Xout, int Mp, int K
         g.upd_decay = (float)(1.0 - fold->lr * fold->weight_decay);
         g.upd_alpha = (float)(-fold->lr);
     }
-    SET_TRACE(g);
+    g.ppx = ppx;
     Timed t(fold ? MUON_HIP_K_BX_UPDATE : MUON_HIP_K_BX, s);
     hipError_t e = launch_gemm_nt(cfg, !fold ? EPI_BX : fold->rows <= fold->cols ? EPI_BX_UPD : EPI_BX_UPD_T, g, s);
     return e == hipSuccess ? 0 : hip_fail(e, "bx launch");
@@ -257,13 +269,6 @@ int dtype_ok(int d) { return d == MUON_HIP_F32 || d == MUON_HIP_BF16; }
 }  // namespace
 
 extern "C" {
-
-#ifdef MUON_TILE_TRACE
-int muon_hip_debug_set_trace(void* buf) {
-    g_trace = (long*)buf;
-    return 0;
-}
-#endif
 
 int muon_hip_version(void) { return 100; }
 
@@ -330,7 +335,8 @@ int muon_hip_normalize(void* workspace, int rows, int cols, int batch, void* str
     Timed t(MUON_HIP_K_NORMALIZE, s);
     hipError_t e = launch_normalize(wsp(workspace, p.offX[1]), p.strideU, (const float*)((char*)workspace + p.offParts),
                                     p.nparts, (float*)((char*)workspace + p.offDenom), wsp(workspace, p.offX[0]),
-                                    p.strideX, rows, cols, p.Mp, p.Kp, batch, s);
+                                    p.strideX, rows, cols, p.Mp, p.Kp, batch, ws_ppx(workspace, p),
+                                    (int)(GEMM_PPX_COUNTER_BYTES / sizeof(unsigned)), s);
     return e == hipSuccess ? 0 : hip_fail(e, "normalize launch");
 }
 
@@ -349,11 +355,12 @@ int ns_chain(void* workspace, int rows, int cols, int batch, int steps, double a
     bf16_t* X[2] = {wsp(workspace, p.offX[0]), wsp(workspace, p.offX[1])};
     bf16_t* A = wsp(workspace, p.offA);
     bf16_t* B = wsp(workspace, p.offB);
+    unsigned* ppx = ws_ppx(workspace, p);  // zero: muon_hip_normalize has just cleared them
     int cur = 0;
     for (int it = 0; it < steps; ++it) {
-        if (int rc = do_syrk(pick_cfg(p.M, EPI_SYRK, p.Kp), X[cur], A, p.Mp, p.Kp, batch, s)) return rc;
-        if (int rc = do_sympoly(pick_cfg(p.M, EPI_SYMPOLY), A, B, p.Mp, batch, b, c, s)) return rc;
-        if (int rc = do_bx(pick_cfg(p.M, EPI_BX), B, X[cur], X[cur ^ 1], p.Mp, p.Kp, batch, a, s,
+        if (int rc = do_syrk(pick_cfg(p.M, EPI_SYRK, p.Kp), X[cur], A, p.Mp, p.Kp, batch, ppx, s)) return rc;
+        if (int rc = do_sympoly(pick_cfg(p.M, EPI_SYMPOLY), A, B, p.Mp, batch, b, c, ppx, s)) return rc;
+        if (int rc = do_bx(pick_cfg(p.M, EPI_BX), B, X[cur], X[cur ^ 1], p.Mp, p.Kp, batch, a, ppx, s,
                            it == steps - 1 ? fold : nullptr))
             return rc;
         cur ^= 1;
@@ -441,30 +448,34 @@ int muon_hip_unpack_bf16(const void* src, int rows_p, int cols_p, void* dst, lon
     return e == hipSuccess ? 0 : hip_fail(e, "unpack launch");
 }
 
-int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* stream) {
+int muon_hip_syrk_bf16(const void* X, void* A, int Mp, int Kp, int batch, int cfg, void* counters, void* stream) {
     if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp, EPI_SYRK, Kp);
     int tile;
     if (int rc = check_gemm(cfg, Mp, Kp, batch, tile)) return rc;
     if (!X || !A) return fail(MUON_HIP_EINVAL, "null operand");
-    return do_syrk(cfg, (const bf16_t*)X, (bf16_t*)A, Mp, Kp, batch, (hipStream_t)stream);
+    if (int rc = check_counters(counters)) return rc;
+    return do_syrk(cfg, (const bf16_t*)X, (bf16_t*)A, Mp, Kp, batch, (unsigned*)counters, (hipStream_t)stream);
 }
 
-int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* stream) {
+int muon_hip_sympoly_bf16(const void* A, void* B, int Mp, int batch, double b, double c, int cfg, void* counters,
+                          void* stream) {
     if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp, EPI_SYMPOLY);
     int tile;
     if (int rc = check_gemm(cfg, Mp, Mp, batch, tile)) return rc;
     if (!A || !B || A == B) return fail(MUON_HIP_EINVAL, "null or aliased operand");
-    return do_sympoly(cfg, (const bf16_t*)A, (bf16_t*)B, Mp, batch, b, c, (hipStream_t)stream);
+    if (int rc = check_counters(counters)) return rc;
+    return do_sympoly(cfg, (const bf16_t*)A, (bf16_t*)B, Mp, batch, b, c, (unsigned*)counters, (hipStream_t)stream);
 }
 
 int muon_hip_bx_axpy_bf16(const void* B, const void* X, void* Xout, int Mp, int Kp, int batch, double a, int cfg,
-                          void* stream) {
+                          void* counters, void* stream) {
     if (cfg == MUON_HIP_CFG_AUTO) cfg = pick_cfg(Mp, EPI_BX);
     int tile;
     if (int rc = check_gemm(cfg, Mp, Kp, batch, tile)) return rc;
     if (!B || !X || !Xout) return fail(MUON_HIP_EINVAL, "null operand");
     if (Xout == X) return fail(MUON_HIP_EINVAL, "Xout must not alias X");
-    return do_bx(cfg, (const bf16_t*)B, (const bf16_t*)X, (bf16_t*)Xout, Mp, Kp, batch, a, (hipStream_t)stream);
+    if (int rc = check_counters(counters)) return rc;
+    return do_bx(cfg, (const bf16_t*)B, (const bf16_t*)X, (bf16_t*)Xout, Mp, Kp, batch, a, (unsigned*)counters, (hipStream_t)stream);
 }
 
 int muon_hip_adamw(void* p, const void* g, void* exp_avg, void* exp_avg_sq, int dtype, long n, int step, double lr,
@@ -609,18 +620,30 @@ int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long
     return e == hipSuccess ? 0 : hip_fail(e, "clip_scale launch");
 }
 
-int muon_hip_mfma_probe(const void* operands, void* sink, int shape, int iters, double* flop, void* stream) {
-    if (!operands || !sink) return fail(MUON_HIP_EINVAL, "null buffer");
-    if ((shape != 0 && shape != 1) || iters <= 0) return fail(MUON_HIP_EINVAL, "shape is 0 or 1 and iters positive");
-    hipError_t e = launch_mfma_probe(operands, (float*)sink, shape, iters, (hipStream_t)stream);
-    if (flop) *flop = MUON_PROBE_FLOP_PER_ITER * iters;
-    return e == hipSuccess ? 0 : hip_fail(e, "mfma_probe launch");
+int muon_hip_device_shape(int* compute_units, int* xcds) {
+    MachineShape ms;
+    if (hipError_t e = machine_shape(ms); e != hipSuccess) return hip_fail(e, "device attributes");
+    if (compute_units) *compute_units = ms.cus;
+    if (xcds) *xcds = 1 << ms.xcd_shift;
+    return 0;
+}
+
+int muon_hip_timing_reserve(long launches) {
+    if (launches < 0 || (size_t)launches > kMaxPool) return fail(MUON_HIP_EINVAL, "0 to %ld launches can be reserved", (long)kMaxPool);
+    if (g_timing.load(std::memory_order_acquire)) return fail(MUON_HIP_EINVAL, "reserve events while timing is off");
+    std::lock_guard<std::mutex> lk(g_tmu);
+    return grow_pool((size_t)launches);
 }
 
 int muon_hip_timing_enable(int on) {
     std::lock_guard<std::mutex> lk(g_tmu);
-    clear_events();
-    g_timing.store(on != 0, std::memory_order_release);
+    g_timing.store(false, std::memory_order_release);
+    if (on) {
+        if (int rc = grow_pool(kPoolChunk)) return rc;  // at least one chunk (a no-op once it exists)
+        g_used.store(0, std::memory_order_relaxed);  // the pairs of the last measurement are recorded over
+        g_untimed.store(0, std::memory_order_relaxed);
+        g_timing.store(true, std::memory_order_release);
+    }
     return 0;
 }
 
@@ -628,18 +651,25 @@ int muon_hip_timing_read(int kernel_id, double* total_ms, long* launches) {
     if (kernel_id < 0 || kernel_id >= MUON_HIP_K_COUNT || !total_ms || !launches)
         return fail(MUON_HIP_EINVAL, "bad kernel id or null output");
     std::lock_guard<std::mutex> lk(g_tmu);
+    const size_t used = std::min(g_used.load(std::memory_order_acquire), g_pool_size.load(std::memory_order_acquire));
     double tot = 0.0;
-    for (auto& p : g_events[kernel_id]) {
+    long cnt = 0;
+    for (size_t i = 0; i < used; ++i) {
+        const EventPair& p = pool_at(i);
+        if (p.kid != kernel_id) continue;
         hipError_t e = hipEventSynchronize(p.stop);
         if (e != hipSuccess) return hip_fail(e, "event synchronize");
         float ms = 0.f;
         e = hipEventElapsedTime(&ms, p.start, p.stop);
         if (e != hipSuccess) return hip_fail(e, "event elapsed");
         tot += ms;
+        ++cnt;
     }
     *total_ms = tot;
-    *launches = (long)g_events[kernel_id].size();
+    *launches = cnt;
     return 0;
 }
+
+long muon_hip_timing_untimed(void) { return g_untimed.load(std::memory_order_relaxed); }
 
 }  // extern "C"

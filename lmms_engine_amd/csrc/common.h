@@ -15,8 +15,6 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 #define MUON_HIP_F32 0
 #define MUON_HIP_BF16 1
 
-#define XCD_COUNT 8
-
 // Every matrix of the Newton-Schulz workspace is stored in blocks of 256 rows x BLK_COLS
 // columns (rows of a block back to back): element (r, c) of a matrix with `cb` column blocks is at
 //   ((r / 256) * cb + c / BLK_COLS) * BLK_ELEMS + (r % 256) * BLK_COLS + c % BLK_COLS.
@@ -58,17 +56,18 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// Workgroups are dealt to the 8 XCDs round-robin by their linear id.  Give each XCD runs of
+// Workgroups are dealt to the XCDs (2^xcd_shift of them) round-robin by their linear id.  Give each XCD runs of
 // XCD_CHUNK consecutive logical ids instead (one round of its 32 CUs), so tiles that share operands
-// share an L2, and deal those runs to the XCDs in turn, so that at any time all eight work on
+// share an L2, and deal those runs to the XCDs in turn, so that at any time all of them work on
 // neighbouring tiles of the same matrix and the memory-side cache, which all XCDs share, serves
 // the panels the others have already fetched.
 #ifndef XCD_CHUNK
 #define XCD_CHUNK 32
 #endif
-__device__ __forceinline__ int xcd_remap(int pid, int nblocks) {
-    const int full = nblocks / (XCD_COUNT * XCD_CHUNK) * (XCD_COUNT * XCD_CHUNK);
+__device__ __forceinline__ int xcd_remap(int pid, int nblocks, int xcd_shift) {
+    const int span = XCD_CHUNK << xcd_shift;  // one run for every XCD
+    const int full = nblocks / span * span;
     if (pid >= full) return pid;
-    const int xcd = pid % XCD_COUNT, local = pid / XCD_COUNT;
-    return ((local / XCD_CHUNK) * XCD_COUNT + xcd) * XCD_CHUNK + local % XCD_CHUNK;
+    const int xcd = pid & ((1 << xcd_shift) - 1), local = pid >> xcd_shift;
+    return (((local / XCD_CHUNK) << xcd_shift) + xcd) * XCD_CHUNK + local % XCD_CHUNK;
 }

@@ -12,7 +12,8 @@ hipError_t launch_momentum_norm(const void* const* g_ptrs, const void* const* m_
 hipError_t launch_cast_norm(const void* G, long strideG, int g_dtype, bf16_t* U, long strideU, float* partials,
                             int nparts, long n, int batch, hipStream_t stream);
 hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, float* denom, bf16_t* X,
-                            long strideX, int rows, int cols, int Mp, int Kp, int batch, hipStream_t stream);
+                            long strideX, int rows, int cols, int Mp, int Kp, int batch, unsigned* clear, int clear_words,
+                            hipStream_t stream);
 hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf16_t* O, long strideO, int cbo,
                                int rows, int cols, int batch, double scale, double lr, double wd,
                                hipStream_t stream);

@@ -189,10 +189,14 @@ cast_norm_kernel(const GT* G, long strideG, bf16_t* U, long strideU, float* part
     if (threadIdx.x == 0) partials[(long)b * gridDim.x + blockIdx.x] = ss;
 }
 
-// d = bf(bf(sqrt(sum)) + 1e-7) per matrix, from its partial sums in a fixed order.
-__global__ void __launch_bounds__(256) frob_finalize_kernel(const float* partials, int nparts, float* denom) {
+// d = bf(bf(sqrt(sum)) + 1e-7) per matrix, from its partial sums in a fixed order.  The first workgroup also clears
+// `clear_words` words at `clear` (the tile counters of the persistent GEMM kernels that follow on the stream).
+__global__ void __launch_bounds__(256) frob_finalize_kernel(const float* partials, int nparts, float* denom,
+                                                            unsigned* clear, int clear_words) {
     __shared__ float red[4];
     const int b = blockIdx.x;
+    if (b == 0 && clear)
+        for (int i = threadIdx.x; i < clear_words; i += 256) clear[i] = 0u;
     float s = 0.f;
     for (int i = threadIdx.x; i < nparts; i += 256) s += partials[(long)b * nparts + i];
     s = block_sum_256(s, red);
@@ -578,8 +582,9 @@ hipError_t launch_cast_norm(const void* G, long strideG, int g_dtype, bf16_t* U,
 }
 
 hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials, int nparts, float* denom, bf16_t* X,
-                            long strideX, int rows, int cols, int Mp, int Kp, int batch, hipStream_t stream) {
-    hipLaunchKernelGGL(frob_finalize_kernel, dim3(batch), dim3(256), 0, stream, partials, nparts, denom);
+                            long strideX, int rows, int cols, int Mp, int Kp, int batch, unsigned* clear, int clear_words,
+                            hipStream_t stream) {
+    hipLaunchKernelGGL(frob_finalize_kernel, dim3(batch), dim3(256), 0, stream, partials, nparts, denom, clear, clear_words);
     // u's padded image is Rp x Cp with Rp a multiple of 64 and Cp a multiple of 128 (both are multiples of the tile edge)
     dim3 grid((Mp / 64) * (Kp / 64) / 2, batch), block(256);
     hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, strideX, rows, cols, Mp, Kp);

@@ -47,13 +47,24 @@ struct GemmArgs {
     int upd_rows, upd_cols;       // the parameter's own (unpadded) shape
     float upd_scale, upd_decay, upd_alpha;  // python-double scale, 1 - lr*wd and -lr, as fp32
     int big_blocks;         // set by the launcher: workgroups that compute whole 256x256 tiles (split-tail kernel)
-    int ppx_slot;           // set by the launcher: which set of tile counters the persistent kernel uses
-#ifdef MUON_TILE_TRACE
-    long* trace;            // measurement builds only: 8 longs per workgroup
-#endif
+    unsigned* ppx;          // tile counters of the persistent kernel (GEMM_PPX_COUNTER_BYTES, zero between launches);
+                            // null: the launcher takes the one-tile kernels instead
+    int xcd_shift;          // set by the launcher: log2 of the XCD count of the device
 };
 
-constexpr int GEMM_CU_COUNT = 256;  // compute units of the part: one 256x256 workgroup each
+// Tile counters of one persistent launch: a 64-byte line per XCD (tiles handed out beyond the two static rounds) and one
+// for the workgroups that have left.  A launch finds them zero and leaves them zero (the last workgroup out resets them),
+// so launches that share a buffer must be ordered on one stream.
+constexpr int GEMM_MAX_XCDS = 8;
+constexpr size_t GEMM_PPX_COUNTER_BYTES = (GEMM_MAX_XCDS + 1) * 16 * sizeof(unsigned);
+
+// Shape of the current device, read once per device: compute units (one 256x256 workgroup each per round of tiles) and
+// XCDs.  gfx950 dies carry 32 active compute units per XCD, and a partition of the part exposes whole XCDs, so the XCD
+// count is the compute-unit count over 32; workgroups are dealt to the XCDs round-robin by their linear id.
+struct MachineShape {
+    int cus, xcd_shift;
+};
+hipError_t machine_shape(MachineShape& ms);
 
 int gemm_cfg_tile(int cfg);
 hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t stream);

@@ -88,28 +88,8 @@ __device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int logical) {
 
 template <int EPI>
 __device__ __forceinline__ TileCoord decode_tile(const GemmArgs& g) {
-    return tile_of<EPI>(g, xcd_remap(blockIdx.x, gridDim.x));
+    return tile_of<EPI>(g, xcd_remap(blockIdx.x, gridDim.x, g.xcd_shift));
 }
-
-// Per-workgroup timestamps for measurement builds (-DMUON_TILE_TRACE): slot 0 entry, 1 operands of the first
-// k-tiles in LDS, 2 end of the k loop, 3 end of the epilogue (100 MHz counter); slots 4, 5: shader-clock count at
-// entry and exit; slot 6: hardware id (which compute unit ran the workgroup).  Compiled out of the product build.
-#ifdef MUON_TILE_TRACE
-#define MUON_TRACE_STAMP(g, slot)                                                                                  \
-    do {                                                                                                           \
-        if ((g).trace && threadIdx.x == 0) {                                                                       \
-            (g).trace[(long)blockIdx.x * 8 + (slot)] = (long)__builtin_amdgcn_s_memrealtime();                      \
-            if ((slot) == 0) {                                                                                     \
-                (g).trace[(long)blockIdx.x * 8 + 4] = (long)__builtin_amdgcn_s_memtime();                          \
-                (g).trace[(long)blockIdx.x * 8 + 6] = (long)__builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)) | \
-                                                     ((long)__builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11)) << 32); \
-            }                                                                                                      \
-            if ((slot) == 3) (g).trace[(long)blockIdx.x * 8 + 5] = (long)__builtin_amdgcn_s_memtime();             \
-        }                                                                                                          \
-    } while (0)
-#else
-#define MUON_TRACE_STAMP(g, slot) do { } while (0)
-#endif
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 typedef const __attribute__((address_space(1))) void* glb_void_ptr;
@@ -936,7 +916,6 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
     WAIT_VM(2 * NLD);
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    MUON_TRACE_STAMP(g, 1);
     if (grp) __builtin_amdgcn_s_barrier();
 
     // LDS read addresses: one register per operand (BX: per half of a piece) and pair of stages; the stage
@@ -1031,7 +1010,6 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
         run_if_mine(std::integral_constant<int, 7>{});
     }
     if (!grp) __builtin_amdgcn_s_barrier();
-    MUON_TRACE_STAMP(g, 2);
     if constexpr (EPI == EPI_BX) {
         // no LDS in this epilogue: the loads issued past the end may land while it runs (its own loads are behind
         // them in the queue, so they have landed before the wave ends)
@@ -1051,9 +1029,7 @@ __device__ __forceinline__ void pp_tile(const GemmArgs& g, const TileCoord& tc, 
 template <int BM, int BN, int WGM, int WGN, int EPI>
 __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArgs g) {
     extern __shared__ __align__(16) unsigned char smem[];
-    MUON_TRACE_STAMP(g, 0);
     pp_tile<BM, BN, WGM, WGN, EPI>(g, decode_tile<EPI>(g), smem);
-    MUON_TRACE_STAMP(g, 3);
 }
 
 // The same with a split tail: when the tile count leaves the last round of the 256 CUs mostly empty,
@@ -1065,7 +1041,7 @@ template <int EPI>
 __global__ void __launch_bounds__(512) gemm_nt_pp_tail_kernel(const GemmArgs g) {
     extern __shared__ __align__(16) unsigned char smem[];
     if ((int)blockIdx.x < g.big_blocks) {
-        pp_tile<256, 256, 2, 4, EPI>(g, tile_of<EPI>(g, xcd_remap(blockIdx.x, g.big_blocks)), smem);
+        pp_tile<256, 256, 2, 4, EPI>(g, tile_of<EPI>(g, xcd_remap(blockIdx.x, g.big_blocks, g.xcd_shift)), smem);
     } else {
         const int s = blockIdx.x - g.big_blocks, quarter = s & 3;
         TileCoord tc = tile_of<EPI>(g, g.big_blocks + (s >> 2));
@@ -1087,31 +1063,14 @@ __global__ void __launch_bounds__(512) gemm_nt_pp_tail_kernel(const GemmArgs g) 
 // Tiles are handed out per XCD, in the order xcd_remap gives a one-tile-per-workgroup launch: workgroup b sits on
 // XCD b % 8 and takes "virtual workgroup ids" 8 n + b % 8.  Its first two n are static (b / 8 and b / 8 + grid / 8),
 // later ones come from an atomic counter of its XCD, asked for during the epilogue of the tile before the one whose
-// last phases need it.  The counters live in a file-scope array (zero when the library is loaded); the last
-// workgroup to leave puts the launch's slot back to zero, launches take slots in turn.
-constexpr int PPX_SLOTS = 64;
+// last phases need it.  The counters are the caller's (GemmArgs::ppx, a piece of the workspace of the call): a launch
+// finds them zero, and the last workgroup to leave puts them back to zero, so the library keeps no state of its own
+// and calls with different workspaces do not meet.
 struct PpxCounters {
-    unsigned next[XCD_COUNT][16];  // a cache line per XCD: tiles handed out beyond the two static rounds
-    unsigned done[16];             // workgroups that have left
+    unsigned next[GEMM_MAX_XCDS][16];  // a cache line per XCD: tiles handed out beyond the two static rounds
+    unsigned done[16];                 // workgroups that have left
 };
-__device__ PpxCounters g_ppx[PPX_SLOTS];
-
-#ifdef MUON_TILE_TRACE
-#define MUON_TRACE_STAMP_AT(g, idx, slot)                                                                          \
-    do {                                                                                                           \
-        if ((g).trace && threadIdx.x == 0) {                                                                       \
-            (g).trace[(long)(idx) * 8 + (slot)] = (long)__builtin_amdgcn_s_memrealtime();                          \
-            if ((slot) == 0) {                                                                                     \
-                (g).trace[(long)(idx) * 8 + 4] = (long)__builtin_amdgcn_s_memtime();                               \
-                (g).trace[(long)(idx) * 8 + 6] = (long)__builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11)) | \
-                                                 ((long)__builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11)) << 32); \
-            }                                                                                                      \
-            if ((slot) == 3) (g).trace[(long)(idx) * 8 + 5] = (long)__builtin_amdgcn_s_memtime();                  \
-        }                                                                                                          \
-    } while (0)
-#else
-#define MUON_TRACE_STAMP_AT(g, idx, slot) do { } while (0)
-#endif
+static_assert(sizeof(PpxCounters) == GEMM_PPX_COUNTER_BYTES, "the size the header promises");
 
 template <int EPI>
 __global__ void __launch_bounds__(512) gemm_nt_ppx_kernel(const GemmArgs g) {
@@ -1133,7 +1092,8 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_kernel(const GemmArgs g) {
     const int wm = wave / WGN, wn = wave % WGN;
     const int kb = g.kdim / BLK_COLS;
     const int total = g.tiles_per_mat * g.batch;
-    const int grid = gridDim.x, xcd = blockIdx.x % XCD_COUNT;
+    const int grid = gridDim.x, xcds = 1 << g.xcd_shift, xcd = blockIdx.x & (xcds - 1);
+    PpxCounters& ctr = *(PpxCounters*)g.ppx;
 
     auto panel_p = [&](const TileCoord& t) { return uniform_ptr(g.P + t.bidx * g.strideP + panel_offset(t.ti * BM, kb)); };
     auto panel_q = [&](const TileCoord& t) {
@@ -1195,24 +1155,22 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_kernel(const GemmArgs g) {
 
     // this workgroup's tiles: the current one, the one after it (virtual ids; >= total means none)
     int pid_cur = blockIdx.x, pid_nxt = blockIdx.x + grid;
-    TileCoord tc = tile_of<EPI>(g, xcd_remap(pid_cur, total));
+    TileCoord tc = tile_of<EPI>(g, xcd_remap(pid_cur, total, g.xcd_shift));
     const bf16_t* Pb = panel_p(tc);
     const bf16_t* Qb = panel_q(tc);
 
-    MUON_TRACE_STAMP_AT(g, pid_cur, 0);
     issue_tile(Pb, Qb, 0);
     issue_tile(Pb, Qb, 1);
     issue_tile(Pb, Qb, 2);
     WAIT_VM(0);  // a tile starts with its k-tiles 0, 1 and 2 in LDS
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    MUON_TRACE_STAMP_AT(g, pid_cur, 1);
     if (grp) __builtin_amdgcn_s_barrier();
 
     for (;;) {
         const bool has_next = pid_nxt < total;
         // without a next tile the last phases load this tile's first k-tiles again, into stages nobody reads any more
-        const TileCoord ntc = has_next ? tile_of<EPI>(g, xcd_remap(pid_nxt, total)) : tc;
+        const TileCoord ntc = has_next ? tile_of<EPI>(g, xcd_remap(pid_nxt, total, g.xcd_shift)) : tc;
         const bf16_t* Pn = panel_p(ntc);
         const bf16_t* Qn = panel_q(ntc);
 
@@ -1295,12 +1253,11 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_kernel(const GemmArgs g) {
             body(nk - 2, I2{}, Yes{}, No{}, No{});
             body(nk - 1, I3{}, Yes{}, No{}, No{});
             if (!grp) __builtin_amdgcn_s_barrier();  // the two groups leave the k loop together
-            MUON_TRACE_STAMP_AT(g, pid_cur, 2);
 
             // Every wave drains its accumulators on its own.  One lane asks for the id of the tile after the next (an
             // increment with wrap-around at 2^32 - 1: a plain atomicAdd of a uniform value is turned into a wave-wide
             // reduction by the compiler, which then waits for the answer on the spot); the answer is needed at the end.
-            if (has_next && tid == 0) fetched = atomicInc(&g_ppx[g.ppx_slot].next[xcd][0], 0xffffffffu);
+            if (has_next && tid == 0) fetched = atomicInc(&ctr.next[xcd][0], 0xffffffffu);
             if constexpr (QT) {
                 epilogue_nn_reg<BM, BN, WGM, WGN>(g, tc, acc);
             } else {
@@ -1337,32 +1294,26 @@ __global__ void __launch_bounds__(512) gemm_nt_ppx_kernel(const GemmArgs g) {
         // (the answer stays untouched until here: any arithmetic on it would be scheduled next to the atomic, with a
         // wait for it)
         asm volatile("" : "+v"(fetched));
-        if (tid == 0) *(int*)(smem + SLOT_OFF) = has_next ? (2 * (grid / XCD_COUNT) + (int)fetched) * XCD_COUNT + xcd : total;
+        if (tid == 0) *(int*)(smem + SLOT_OFF) = has_next ? (((2 * (grid >> g.xcd_shift) + (int)fetched)) << g.xcd_shift) + xcd : total;
         // The loads of the epilogue are behind those of the next tile's first k-tiles in the queue and have been
         // consumed, so every wave's share of those k-tiles has landed: publish them, and the id.
         __syncthreads();
-        MUON_TRACE_STAMP_AT(g, pid_cur, 3);
         if (!has_next) break;
         pid_cur = pid_nxt;
         pid_nxt = __builtin_amdgcn_readfirstlane(*(const int*)(smem + SLOT_OFF));
         tc = ntc;
         Pb = Pn;
         Qb = Qn;
-        MUON_TRACE_STAMP_AT(g, pid_cur, 0);
-        MUON_TRACE_STAMP_AT(g, pid_cur, 1);
         if (grp) __builtin_amdgcn_s_barrier();  // and enter the next tile a phase apart again
     }
     if (tid == 0) {
-        PpxCounters& c = g_ppx[g.ppx_slot];
         // every workgroup has its last answer from `next` before it counts itself out, so the last one out may reset
-        if (atomicAdd(&c.done[0], 1u) == (unsigned)grid - 1) {
-            for (int x = 0; x < XCD_COUNT; ++x) atomicExch(&c.next[x][0], 0u);
-            atomicExch(&c.done[0], 0u);
+        if (atomicAdd(&ctr.done[0], 1u) == (unsigned)grid - 1) {
+            for (int x = 0; x < xcds; ++x) atomicExch(&ctr.next[x][0], 0u);
+            atomicExch(&ctr.done[0], 0u);
         }
     }
 }
-
-std::atomic<unsigned> g_ppx_sequence{0};  // launches take the counter slots in turn
 
 // Dynamic LDS beyond 64 KB has to be allowed per kernel, and the attribute belongs to the device that is current when
 // it is set: once per (kernel instantiation, device), remembered as one bit per device in the instantiation's mask.
@@ -1379,12 +1330,11 @@ hipError_t allow_dynamic_lds(const void* kern, int bytes, std::atomic<unsigned l
 }
 
 template <int EPI>
-hipError_t launch_ppx(GemmArgs g, int nblocks, hipStream_t stream) {
+hipError_t launch_ppx(const GemmArgs& g, int nblocks, int cus, hipStream_t stream) {
     constexpr int smem = 4 * (256 + 256) * 64 + 64;
     static std::atomic<unsigned long long> configured{0};  // per instantiation
     if (hipError_t e = allow_dynamic_lds((const void*)gemm_nt_ppx_kernel<EPI>, smem, configured); e != hipSuccess) return e;
-    g.ppx_slot = (int)(g_ppx_sequence.fetch_add(1, std::memory_order_relaxed) % PPX_SLOTS);
-    const int grid = nblocks < GEMM_CU_COUNT ? nblocks : GEMM_CU_COUNT;
+    const int grid = nblocks < cus ? nblocks : cus;  // a whole number of XCDs: the caller launches more tiles than CUs
     hipLaunchKernelGGL(gemm_nt_ppx_kernel<EPI>, dim3(grid), dim3(512), smem, stream, g);
     return hipGetLastError();
 }
@@ -1446,22 +1396,45 @@ hipError_t launch_pp_tail(GemmArgs g, int nblocks, int rest, hipStream_t stream)
 #ifndef PPX_SYMPOLY_MAXK
 #define PPX_SYMPOLY_MAXK 2048
 #endif
-hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& g, hipStream_t stream) {
+hipError_t machine_shape(MachineShape& ms) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cached[kMaxDevices];  // compute units per device ordinal, 0 = not read yet
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    int cus = (dev >= 0 && dev < kMaxDevices) ? cached[dev].load(std::memory_order_relaxed) : 0;
+    if (cus == 0) {
+        if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev); e != hipSuccess) return e;
+        if (cus <= 0) return hipErrorInvalidDevice;
+        if (dev >= 0 && dev < kMaxDevices) cached[dev].store(cus, std::memory_order_relaxed);
+    }
+    ms.cus = cus;
+    int xcds = cus / 32;  // 32 active compute units per XCD on gfx950
+    ms.xcd_shift = 0;
+    while ((2 << ms.xcd_shift) <= xcds && (2 << ms.xcd_shift) <= GEMM_MAX_XCDS && cus % (2 << ms.xcd_shift) == 0) ++ms.xcd_shift;
+    return hipSuccess;
+}
+
+hipError_t launch_gemm_nt(int cfg, int epi, const GemmArgs& args, hipStream_t stream) {
+    GemmArgs g = args;
+    MachineShape ms;
+    if (hipError_t e = machine_shape(ms); e != hipSuccess) return e;
+    g.xcd_shift = ms.xcd_shift;
+    const int cus = ms.cus;
     const int nblocks = g.tiles_per_mat * g.batch;
     if (nblocks <= 0) return hipSuccess;
     // Ping-pong kernel: split the tiles of a last round that would fill at most a quarter of the CUs (a 128x128
     // tile takes about 0.6 of the time of a 256x256 one, so one round of quarters beats a round of whole tiles).
-    const int rest = nblocks % GEMM_CU_COUNT;
+    const int rest = nblocks % cus;
     if (cfg == GEMM_CFG_256_PERSIST) {
-        // a.X + B.X with at least 8 k-tiles and more tiles than compute units; everything else takes the one-tile kernel
-        if (g.kdim >= 256 && nblocks > GEMM_CU_COUNT) {
-            if (epi == EPI_BX) return launch_ppx<EPI_BX>(g, nblocks, stream);
-            if (epi == EPI_SYRK && g.kdim <= PPX_SYRK_MAXK) return launch_ppx<EPI_SYRK>(g, nblocks, stream);
-            if (epi == EPI_SYMPOLY && g.kdim <= PPX_SYMPOLY_MAXK) return launch_ppx<EPI_SYMPOLY>(g, nblocks, stream);
+        // at least 8 k-tiles, more tiles than compute units and a counter buffer; everything else takes the one-tile kernel
+        if (g.kdim >= 256 && nblocks > cus && g.ppx) {
+            if (epi == EPI_BX) return launch_ppx<EPI_BX>(g, nblocks, cus, stream);
+            if (epi == EPI_SYRK && g.kdim <= PPX_SYRK_MAXK) return launch_ppx<EPI_SYRK>(g, nblocks, cus, stream);
+            if (epi == EPI_SYMPOLY && g.kdim <= PPX_SYMPOLY_MAXK) return launch_ppx<EPI_SYMPOLY>(g, nblocks, cus, stream);
         }
         cfg = GEMM_CFG_256_PINGPONG;
     }
-    if (cfg == GEMM_CFG_256_PINGPONG && nblocks > GEMM_CU_COUNT && rest > 0 && rest <= GEMM_CU_COUNT / 4) {
+    if (cfg == GEMM_CFG_256_PINGPONG && nblocks > cus && rest > 0 && rest <= cus / 4) {
         switch (epi) {
             case EPI_SYRK: return launch_pp_tail<EPI_SYRK>(g, nblocks, rest, stream);
             case EPI_SYMPOLY: return launch_pp_tail<EPI_SYMPOLY>(g, nblocks, rest, stream);

@@ -1,9 +1,13 @@
-// Measurement kernels, no part of the optimizer step: loops of nothing but MFMAs on caller-supplied operands.
+// Measurement kernels, no part of the optimizer step and no part of libmuon_hip.so: this file is built into a library of
+// its own (libmuon_probe.so) that only the benchmark's operand-power legs load.  Loops of nothing but MFMAs on
+// caller-supplied operands.
 // They show what the matrix pipes sustain under the part's power management for a given instruction shape and
 // operand content (random mantissas against constants), which is the ceiling the Newton-Schulz GEMMs are
 // measured against and the reason they are built on v_mfma_f32_16x16x32_bf16.
 #include "common.h"
-#include "probe.h"
+
+#define MUON_PROBE_BLOCKS 256                            // workgroups: one per compute unit of a whole part
+#define MUON_PROBE_FLOP_PER_ITER (256.0 * 8 * 16 * 32768.0)
 
 namespace {
 
@@ -69,10 +73,16 @@ __global__ void __launch_bounds__(512) mfma_probe_kernel(const bf16x8* src, floa
 
 }  // namespace
 
-hipError_t launch_mfma_probe(const void* operands, float* sink, int shape, int iters, hipStream_t stream) {
+// shape 0: v_mfma_f32_32x32x16_bf16, shape 1: v_mfma_f32_16x16x32_bf16.  `operands` holds 256 * 12 * 512 * 16 bytes of
+// bf16 values chosen by the caller (random, constant ...), `sink` receives 256 * 512 floats; *flop is the work of the
+// launch.  Returns a hipError_t (0 = launched) or -1 for bad arguments.  Time it with events on `stream`.
+extern "C" __attribute__((visibility("default"))) int muon_probe_mfma(const void* operands, void* sink, int shape, int iters,
+                                                                      double* flop, void* stream) {
+    if (!operands || !sink || (shape != 0 && shape != 1) || iters <= 0) return -1;
     dim3 grid(MUON_PROBE_BLOCKS), block(512);
-    if (shape == 0) hipLaunchKernelGGL(mfma_probe_kernel<0>, grid, block, 0, stream, (const bf16x8*)operands, sink, iters);
-    else if (shape == 1) hipLaunchKernelGGL(mfma_probe_kernel<1>, grid, block, 0, stream, (const bf16x8*)operands, sink, iters);
-    else return hipErrorInvalidValue;
-    return hipGetLastError();
+    hipStream_t s = (hipStream_t)stream;
+    if (shape == 0) hipLaunchKernelGGL(mfma_probe_kernel<0>, grid, block, 0, s, (const bf16x8*)operands, (float*)sink, iters);
+    else hipLaunchKernelGGL(mfma_probe_kernel<1>, grid, block, 0, s, (const bf16x8*)operands, (float*)sink, iters);
+    if (flop) *flop = MUON_PROBE_FLOP_PER_ITER * iters;
+    return (int)hipGetLastError();
 }

@@ -85,9 +85,23 @@ def _pointer_table(tensors, device, cache=None, key=None) -> Tensor:
         hit = cache.get(key)
         if hit is not None and hit[0] == ptrs and hit[1].device == device:
             return hit[1]
+    if torch.cuda.is_current_stream_capturing():
+        # A miss under capture would record a copy out of a host buffer that is freed when this call returns, and
+        # replace a table that an earlier recording may still read.
+        raise _abi.MuonHipError(
+            "Muon.step under HIP graph capture needs the pointer tables of an earlier eager step: parameters, grads "
+            "and momentum buffers must keep their addresses (run an eager step first and do not re-allocate grads, "
+            "e.g. zero_grad(set_to_none=False))"
+        )
     host = torch.tensor(ptrs, dtype=torch.int64, pin_memory=True)
     table = host.to(device, non_blocking=True)
     if cache is not None:
+        old = cache.get(key)
+        if old is not None:
+            # a graph recorded earlier may still read the old table: keep it alive instead of handing its memory
+            # back to the allocator (bounded: one generation per change of addresses)
+            cache.setdefault("_retired", []).append(old[1])
+            del cache["_retired"][:-64]
         cache[key] = (ptrs, table)
     return table
 
@@ -126,7 +140,7 @@ def matmul_transpose_assign(d_in: Tensor, d_out: Tensor) -> None:
         x = torch.empty(lib.muon_hip_blocked_elems(Mp, Kp), dtype=torch.bfloat16, device=d_in.device)
         a = torch.empty(lib.muon_hip_blocked_elems(Mp, Mp), dtype=torch.bfloat16, device=d_in.device)
         _abi.check(lib.muon_hip_pack_bf16(src.data_ptr(), 0, K, M, K, x.data_ptr(), Mp, Kp, 1, s), "pack")
-        _abi.check(lib.muon_hip_syrk_bf16(x.data_ptr(), a.data_ptr(), Mp, Kp, 1, cfg, s), "syrk")
+        _abi.check(lib.muon_hip_syrk_bf16(x.data_ptr(), a.data_ptr(), Mp, Kp, 1, cfg, None, s), "syrk")
         out = d_out if d_out.is_contiguous() else torch.empty_like(d_out, memory_format=torch.contiguous_format)
         _abi.check(lib.muon_hip_unpack_bf16(a.data_ptr(), Mp, Mp, out.data_ptr(), 0, M, M, M, 1, s), "unpack")
         if out is not d_out:
@@ -261,15 +275,24 @@ def muon_update(grad, momentum, beta=0.95, ns_steps=5, nesterov=True, rms_scale=
 # --------------------------------------------------------------------------------------
 # grouped launcher
 # --------------------------------------------------------------------------------------
-_CU_COUNT = 256  # one 256x256 GEMM workgroup per compute unit and round
+_cu_counts = {}  # device index -> compute units, as the library reads them from the runtime
 
 
-def _pick_chunk(n: int, cap: int, rows: int, cols: int) -> int:
-    """Matrices per grouped launch for a bucket of n: about `cap` (what the workspace limit holds; up to an eighth
-    more when that lands on whole rounds), chosen so that the tile counts of the three products leave the last
-    round of the 256 compute units as full as possible.  A launch of t tiles runs ceil(t / 256) rounds (a last
+def _cu_count(device) -> int:
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx not in _cu_counts:
+        with torch.cuda.device(idx):
+            _cu_counts[idx] = _abi.device_shape()[0]
+    return _cu_counts[idx]
+
+
+def _pick_chunk(n: int, cap: int, rows: int, cols: int, cus: int = 256) -> int:
+    """Matrices per grouped launch for a bucket of n: at most `cap` (what the workspace limit holds, and never more
+    than the 65535 matrices one library call takes) and at least half of it, chosen so that the tile counts of the
+    three products leave the last round of the `cus` compute units (one 256x256 workgroup each) as full as possible.  A launch of t tiles runs ceil(t / cus) rounds (a last
     round of at most 64 tiles is cut into quarter tiles and costs about 0.6 of a round) plus about a third of a
     round of ramp-up and tail; a tile of X.Xt costs ~K, one of b.A + c.A.A and of a.X + B.X ~M."""
+    cap = min(cap, 65535)
     if cap >= n or cap <= 2:
         return max(1, min(n, cap))
     M, K = min(rows, cols), max(rows, cols)
@@ -279,14 +302,14 @@ def _pick_chunk(n: int, cap: int, rows: int, cols: int) -> int:
     tri, rect = T * (T + 1) // 2, T * TN
 
     def rounds(t):
-        full, rest = divmod(t, _CU_COUNT)
-        return full + (0.0 if rest == 0 else 0.6 if rest <= _CU_COUNT // 4 and full > 0 else 1.0)
+        full, rest = divmod(t, cus)
+        return full + (0.0 if rest == 0 else 0.6 if rest <= cus // 4 and full > 0 else 1.0)
 
     def cost(nb):
         return (rounds(tri * nb) + 0.35) * (K + M) + (rounds(rect * nb) + 0.35) * M
 
     best, best_cost = cap, None
-    for nb in range(max(1, cap // 2), min(n, cap + cap // 8) + 1):
+    for nb in range(max(1, cap // 2), min(n, cap) + 1):
         chunks, last = divmod(n, nb)
         c = chunks * cost(nb) + (cost(last) if last else 0.0)
         if best_cost is None or c < best_cost * (1 - 1e-9):
@@ -305,7 +328,7 @@ def _muon_bucket_step(params, grads, moms, group, ns_steps, nesterov, write_back
     scale = scale_factor(rows, cols, group["rms_scale"])
     n = len(params)
     per = _abi.workspace_bytes(rows, cols, 1)
-    chunk = _pick_chunk(n, max(1, min(ws_limit // per, 65535)), rows, cols)
+    chunk = _pick_chunk(n, max(1, min(ws_limit // per, 65535)), rows, cols, _cu_count(dev))
     with torch.cuda.device(dev):
         s = _abi.stream_ptr(dev)
         for lo in range(0, n, chunk):

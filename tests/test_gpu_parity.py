@@ -27,7 +27,10 @@ def env():
 
     lib = _abi.lib()  # raises if libmuon_hip.so is missing
     assert lib.muon_hip_version() >= 100
-    return dict(abi=_abi, mu=muon_utils, O=muon_oracle, lib=lib, dev=torch.device("cuda:0"))
+    dev = torch.device("cuda:0")
+    # tile counters for the single-GEMM entry points: zero before the first use, left zero by every launch
+    ctr = torch.zeros(_abi.PPX_COUNTER_BYTES, dtype=torch.uint8, device=dev)
+    return dict(abi=_abi, mu=muon_utils, O=muon_oracle, lib=lib, dev=dev, ctr=ctr, ctr_ptr=ctr.data_ptr())
 
 
 def _ulp_diff_bf16(a: torch.Tensor, b: torch.Tensor) -> int:
@@ -109,7 +112,7 @@ def test_syrk_matches_fp64_and_is_symmetric(env, cfg, M, K, batch):
     X = torch.randn(batch, M, K, generator=g).bfloat16()
     Xb = _pack(env, X.to(env["dev"]))
     Ab = _blocked_nan(env, batch, M, M)
-    env["abi"].check(env["lib"].muon_hip_syrk_bf16(Xb.data_ptr(), Ab.data_ptr(), M, K, batch, cfg, 0))
+    env["abi"].check(env["lib"].muon_hip_syrk_bf16(Xb.data_ptr(), Ab.data_ptr(), M, K, batch, cfg, env["ctr_ptr"], 0))
     A = _unpack(env, Ab, batch, M, M)
     assert torch.equal(A, A.mT), "X·Xᵀ must be symmetric bit for bit"
     ref64 = (X.double() @ X.double().mT)
@@ -128,7 +131,7 @@ def test_sympoly_rounding_points(env, cfg):
     Ab = _pack(env, A.to(env["dev"]))
     Bb = _blocked_nan(env, batch, M, M)
     a, b, c = O.NS_COEFFS
-    env["abi"].check(env["lib"].muon_hip_sympoly_bf16(Ab.data_ptr(), Bb.data_ptr(), M, batch, b, c, cfg, 0))
+    env["abi"].check(env["lib"].muon_hip_sympoly_bf16(Ab.data_ptr(), Bb.data_ptr(), M, batch, b, c, cfg, env["ctr_ptr"], 0))
     B = _unpack(env, Bb, batch, M, M)
     assert torch.equal(B, B.mT)
     for i in range(batch):
@@ -153,7 +156,7 @@ def test_bx_axpy_rounding_points(env, cfg, M, K):
     dev = env["dev"]
     Xb, Bb, Xo = _pack(env, X.to(dev)), _pack(env, Bm.to(dev)), _blocked_nan(env, batch, M, K)
     a = O.NS_COEFFS[0]
-    env["abi"].check(env["lib"].muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, a, cfg, 0))
+    env["abi"].check(env["lib"].muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, a, cfg, env["ctr_ptr"], 0))
     Xo = _unpack(env, Xo, batch, M, K)
     for i in range(batch):
         ref = (O.bf(X[i].float() * O._f32(a)) + O.bf(Bm[i].float() @ X[i].float())).bfloat16()
@@ -173,8 +176,8 @@ def test_split_tail_is_bitwise_the_plain_kernel(env):
     outs = []
     for cfg in (abi.CFG_256_PINGPONG, abi.CFG_256_PIPE):
         Ab, Bb = _blocked_nan(env, batch, M, M), _blocked_nan(env, batch, M, M)
-        abi.check(lib.muon_hip_syrk_bf16(Xb.data_ptr(), Ab.data_ptr(), M, K, batch, cfg, 0))
-        abi.check(lib.muon_hip_sympoly_bf16(Ab.data_ptr(), Bb.data_ptr(), M, batch, O.NS_COEFFS[1], O.NS_COEFFS[2], cfg, 0))
+        abi.check(lib.muon_hip_syrk_bf16(Xb.data_ptr(), Ab.data_ptr(), M, K, batch, cfg, env["ctr_ptr"], 0))
+        abi.check(lib.muon_hip_sympoly_bf16(Ab.data_ptr(), Bb.data_ptr(), M, batch, O.NS_COEFFS[1], O.NS_COEFFS[2], cfg, env["ctr_ptr"], 0))
         outs.append((_unpack(env, Ab, batch, M, M), _unpack(env, Bb, batch, M, M)))
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
     assert torch.equal(outs[0][0], outs[0][0].mT) and not torch.isnan(outs[0][1]).any()
@@ -185,7 +188,7 @@ def test_split_tail_is_bitwise_the_plain_kernel(env):
     outs = []
     for cfg in (abi.CFG_256_PINGPONG, abi.CFG_256_PIPE):
         Xo = _blocked_nan(env, batch, M, K)
-        abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, O.NS_COEFFS[0], cfg, 0))
+        abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, O.NS_COEFFS[0], cfg, env["ctr_ptr"], 0))
         outs.append(_unpack(env, Xo, batch, M, K))
     assert torch.equal(outs[0], outs[1]) and not torch.isnan(outs[0]).any()
 
@@ -209,12 +212,18 @@ def test_persistent_bx_is_bitwise_the_one_tile_kernel(env):
         res = []
         for cfg in (abi.CFG_256_PIPE, abi.CFG_256_PERSIST, abi.CFG_256_PERSIST, abi.CFG_256_PERSIST):
             Xo = _blocked_nan(env, batch, M, K)
-            abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, a_c, cfg, 0))
+            abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, a_c, cfg, env["ctr_ptr"], 0))
             torch.cuda.synchronize()
+            assert not env["ctr"].any(), "a persistent launch leaves its tile counters zero"
             res.append(Xo.clone())
         for rep in (1, 2, 3):
             assert not torch.isnan(res[rep].float()).any(), rep
             assert torch.equal(res[0], res[rep]), f"M={M} K={K} batch={batch}, launch {rep}"
+        # without a counter buffer the same configuration runs the one-tile kernels
+        Xo = _blocked_nan(env, batch, M, K)
+        abi.check(lib.muon_hip_bx_axpy_bf16(Bb.data_ptr(), Xb.data_ptr(), Xo.data_ptr(), M, K, batch, a_c, abi.CFG_256_PERSIST, None, 0))
+        torch.cuda.synchronize()
+        assert torch.equal(res[0], Xo)
 
 
 def test_persistent_symmetric_products_are_bitwise_the_two_stage_kernel(env):
@@ -234,9 +243,10 @@ def test_persistent_symmetric_products_are_bitwise_the_two_stage_kernel(env):
         for cfg in (abi.CFG_256_PIPE, abi.CFG_256_PINGPONG, abi.CFG_256_PERSIST, abi.CFG_256_PERSIST, abi.CFG_256_PERSIST):
             A = _blocked_nan(env, batch, M, M)
             B = _blocked_nan(env, batch, M, M)
-            abi.check(lib.muon_hip_syrk_bf16(Xb.data_ptr(), A.data_ptr(), M, K, batch, cfg, 0))
-            abi.check(lib.muon_hip_sympoly_bf16(A.data_ptr(), B.data_ptr(), M, batch, b_c, c_c, cfg, 0))
+            abi.check(lib.muon_hip_syrk_bf16(Xb.data_ptr(), A.data_ptr(), M, K, batch, cfg, env["ctr_ptr"], 0))
+            abi.check(lib.muon_hip_sympoly_bf16(A.data_ptr(), B.data_ptr(), M, batch, b_c, c_c, cfg, env["ctr_ptr"], 0))
             torch.cuda.synchronize()
+            assert not env["ctr"].any(), "a persistent launch leaves its tile counters zero"
             res.append((A.clone(), B.clone()))
         for rep in (1, 2, 3, 4):  # the one-tile ping-pong kernel, then the persistent one three times
             for name, ref, got in (("syrk", res[0][0], res[rep][0]), ("sympoly", res[0][1], res[rep][1])):
@@ -249,14 +259,14 @@ def test_persistent_symmetric_products_are_bitwise_the_two_stage_kernel(env):
 def test_gemm_entry_points_reject_bad_shapes(env):
     lib, abi = env["lib"], env["abi"]
     x = torch.zeros(256 * 256, dtype=torch.bfloat16, device=env["dev"])
-    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 200, 256, 1, 0, 0) == -2
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 200, 256, 1, 0, env["ctr_ptr"], 0) == -2
     assert b"multiples" in lib.muon_hip_last_error()
-    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 128, 128, 1, abi.CFG_256_PIPE, 0) == -2  # 128 is not a 256-tile
-    assert lib.muon_hip_syrk_bf16(None, x.data_ptr(), 256, 256, 1, 0, 0) == -1
-    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 256, 256, 1, 99, 0) == -1
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 128, 128, 1, abi.CFG_256_PIPE, env["ctr_ptr"], 0) == -2  # 128 is not a 256-tile
+    assert lib.muon_hip_syrk_bf16(None, x.data_ptr(), 256, 256, 1, 0, env["ctr_ptr"], 0) == -1
+    assert lib.muon_hip_syrk_bf16(x.data_ptr(), x.data_ptr(), 256, 256, 1, 99, env["ctr_ptr"], 0) == -1
     with pytest.raises(abi.MuonHipError):
-        abi.check(lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), None, 256, 256, 1, 1.0, 0, 0))
-    assert lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), x.data_ptr(), 256, 256, 1, 1.0, 0, 0) == -1  # in place
+        abi.check(lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), None, 256, 256, 1, 1.0, 0, env["ctr_ptr"], 0))
+    assert lib.muon_hip_bx_axpy_bf16(x.data_ptr(), x.data_ptr(), x.data_ptr(), 256, 256, 1, 1.0, 0, env["ctr_ptr"], 0) == -1  # in place
 
 
 NS_SHAPES = [(64, 160), (160, 64), (33, 47), (100, 300), (300, 100), (128, 896), (896, 128), (256, 256), (512, 1024)]
@@ -649,6 +659,104 @@ def test_grouped_equals_per_matrix_bitwise_on_256_tiles(env):
         assert torch.equal(p.detach(), q.detach()), name
 
 
+def _chunk_plan(env, rows, cols, n, cap):
+    """(workspace limit that holds `cap` matrices of the shape, matrices per launch the optimizer then takes)."""
+    per = env["abi"].workspace_bytes(rows, cols, 1)
+    limit = cap * per + per // 2
+    assert limit // per == cap
+    return limit, env["mu"]._pick_chunk(n, cap, rows, cols)
+
+
+@pytest.mark.parametrize("rows,cols,n,cap,kernel", [
+    (2048, 2048, 23, 8, "persistent"),   # 36 + 36 + 64 tiles a matrix: all three products of a chunk of 8 walk tiles
+    (2048, 1024, 7, 3, "transposed"),    # rows > cols on 256-tiles: the update goes through the transposing gather
+    (640, 384, 10, 4, "128-tiles"),      # short side no whole number of 256-tiles, transposed and ragged
+])
+def test_chunked_bucket_equals_the_unchunked_twin_bitwise(env, rows, cols, n, cap, kernel):
+    """The reference steps one parameter at a time (muon_utils.py:443-456); here a bucket larger than the workspace
+    limit is cut into chunks that share one workspace, each with a cached device pointer table keyed by its first
+    index.  A bucket of n same-shape matrices under a limit that holds `cap` of them must run as at least three chunks
+    with a ragged last one and leave parameters and momentum bit-equal to a twin that runs the bucket in one launch,
+    over three steps (the second and third find the tables of the step before), and within the parity bounds of the
+    CPU oracle on the first, a middle and the last matrix.  The workspace never exceeds the limit."""
+    print(f"chunked dispatch {rows}x{cols} x{n}, cap {cap} ({kernel})", flush=True)
+    mu, O, dev = env["mu"], env["O"], env["dev"]
+    limit, chunk = _chunk_plan(env, rows, cols, n, cap)
+    nchunks = -(-n // chunk)
+    assert nchunks >= 3 and n % chunk != 0, (chunk, nchunks)
+    if kernel == "persistent":
+        T = rows // 256
+        assert chunk * T * (T + 1) // 2 > 256 and chunk * T * (cols // 256) > 256  # more tiles than compute units
+    gen = torch.Generator().manual_seed(rows + 3 * cols + n)
+    w0 = [(0.02 * torch.randn(rows, cols, generator=gen)).bfloat16() for _ in range(n)]
+    hp = dict(MUON_HP)
+    twins = []
+    for lim in (limit, 1 << 40):
+        ps = [torch.nn.Parameter(w.clone().to(dev)) for w in w0]
+        twins.append((ps, mu.Muon([dict(params=list(ps), use_muon=True, **hp)], momentum_dtype=torch.float32,
+                                  workspace_limit_bytes=lim)))
+    sample = sorted({0, n // 2, n - 1})
+    cw = {i: w0[i].clone() for i in sample}
+    cm = {i: torch.zeros(rows, cols) for i in sample}
+    for step in range(3):
+        grads = [(1e-3 * torch.randn(rows, cols, generator=gen)).bfloat16() for _ in range(n)]
+        for ps, opt in twins:
+            for p, g in zip(ps, grads):
+                p.grad = g.to(dev)
+            opt.step()
+        torch.cuda.synchronize()
+        (pa, oa), (pb, ob) = twins
+        assert len(oa._pointer_tables) - ("_retired" in oa._pointer_tables) == nchunks
+        assert oa._workspaces[dev].numel() <= limit < ob._workspaces[dev].numel()
+        for i in range(n):
+            assert torch.equal(pa[i].detach(), pb[i].detach()), f"step {step}, matrix {i}: parameter"
+            assert torch.equal(oa.state[pa[i]]["momentum_buffer"], ob.state[pb[i]]["momentum_buffer"]), f"step {step}, matrix {i}: momentum"
+        sc = O._f32(mu.scale_factor(rows, cols, False))
+        for i in sample:
+            # the orthogonalised update itself: the stage entry points on the same gradient and the momentum before the step
+            got = _ns_via_stages(env, [grads[i].to(dev)], [cm[i].to(dev)])[0]
+            o = O.muon_step_matrix(cw[i], grads[i].clone(), cm[i], lr=hp["lr"], weight_decay=hp["weight_decay"],
+                                   beta=hp["momentum"], nesterov=True, ns_steps=5, rms_scale=False)
+            wu, wm = rel_fro((got.float() * sc).bfloat16(), o), rel_fro(oa.state[pa[i]]["momentum_buffer"], cm[i])
+            report_parity(f"chunked dispatch {rows}x{cols} step {step} matrix {i}: update {wu:.3e} momentum {wm:.3e}")
+            assert wu <= NS_TOL and wm <= MOM_TOL
+            assert rel_fro(pa[i].detach(), cw[i]) <= 4e-3
+
+
+def test_chunked_bucket_follows_a_group_whose_tensors_change(env):
+    """A cached pointer table must miss when the tensors behind a chunk change: between steps one parameter leaves the
+    group (every later matrix moves up one place, across chunk boundaries), the gradients move to fresh addresses, and
+    the parameter comes back.  The chunked optimizer stays bit-equal to the twin that runs one launch per bucket."""
+    mu, dev = env["mu"], env["dev"]
+    rows, cols, n, cap = 512, 768, 11, 4
+    limit, chunk = _chunk_plan(env, rows, cols, n, cap)
+    assert -(-n // chunk) >= 3
+    gen = torch.Generator().manual_seed(77)
+    w0 = [(0.02 * torch.randn(rows, cols, generator=gen)) for _ in range(n)]
+    twins = []
+    for lim in (limit, 1 << 40):
+        ps = [torch.nn.Parameter(w.clone().to(dev)) for w in w0]
+        twins.append((ps, mu.Muon([dict(params=list(ps), use_muon=True, **MUON_HP)], workspace_limit_bytes=lim)))
+    keep = []  # old gradients stay alive, so that new ones cannot land on their addresses
+    members = [list(range(n)), [i for i in range(n) if i != 2], list(range(n)), list(reversed(range(n)))]
+    for step, idx in enumerate(members):
+        grads = [1e-3 * torch.randn(rows, cols, generator=gen) for _ in range(n)]
+        for ps, opt in twins:
+            opt.param_groups[0]["params"] = [ps[i] for i in idx]
+            for p, g in zip(ps, grads):
+                p.grad = g.to(dev)
+                keep.append(p.grad)
+            opt.step()
+        torch.cuda.synchronize()
+        (pa, oa), (pb, ob) = twins
+        for i in range(n):
+            assert torch.equal(pa[i].detach(), pb[i].detach()), f"step {step}, matrix {i}"
+            if pa[i] in oa.state:
+                assert torch.equal(oa.state[pa[i]]["momentum_buffer"], ob.state[pb[i]]["momentum_buffer"])
+    # matrix 2 sat out one step: it differs from a matrix that took all four, i.e. the steps really followed `members`
+    assert not torch.equal(twins[0][0][2].detach(), w0[2].to(dev))
+
+
 BUCKET_SHAPES = [(4096, 4096), (1024, 4096), (12288, 4096), (4096, 12288),      # Qwen3-8B (benchmark config 3)
                  (768, 2048), (2048, 768), (512, 2048), (4096, 2048), (2048, 4096)]  # Qwen3-MoE-30B-A3B (config 5)
 
@@ -800,6 +908,73 @@ def test_muon_step_replays_from_a_hip_graph(env):
         for i, (p, q) in enumerate(zip(pa, pb)):
             assert torch.equal(p, q), (rep, i, shapes[i])
             assert torch.equal(oa.state[p]["momentum_buffer"], ob.state[q]["momentum_buffer"]), (rep, i)
+
+
+def test_two_optimizers_on_two_streams_one_replaying_a_graph(env):
+    """Two optimizers step at the same time on two streams, one of them replaying a recorded HIP graph: everything their
+    kernels share (operands, norms, the tile counters of the persistent kernels) lives in each optimizer's own
+    workspace, so neither can take the other's tiles.  Three rounds, no synchronisation between the two streams inside
+    a round; parameters and momentum must equal those of twins that run the same steps one after the other.  Buckets:
+    expert-shaped matrices (all three products persistent), a transposed one, a 128-tile one."""
+    dev, mu = env["dev"], env["mu"]
+    shapes = [(768, 2048)] * 60 + [(1024, 512)] * 4 + [(384, 640)] * 3
+
+    def make(seed):
+        g = torch.Generator().manual_seed(seed)
+        ps = [torch.nn.Parameter((torch.randn(r, c, generator=g) * 0.02).bfloat16().to(dev)) for r, c in shapes]
+        for p in ps:
+            p.grad = (torch.randn(p.shape, generator=g) * 0.01).bfloat16().to(dev)
+        opt = mu.Muon([dict(params=ps, use_muon=True, lr=0.02, momentum=0.95, weight_decay=0.01, rms_scale=False)],
+                      momentum_dtype=torch.float32)
+        return ps, opt
+
+    # (a, b) run concurrently, a from a graph; (c, d) are their serial twins
+    (pa, oa), (pb, ob), (pc, oc), (pd, od) = make(5), make(6), make(5), make(6)
+    for _ in range(2):
+        for o in (oa, ob, oc, od):
+            o.step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        oa.step()
+    s1, s2 = torch.cuda.Stream(dev), torch.cuda.Stream(dev)
+    for rep in range(3):
+        print(f"two streams, round {rep}", flush=True)
+        with torch.cuda.stream(s1):
+            graph.replay()
+        with torch.cuda.stream(s2):
+            ob.step()
+        oc.step()
+        od.step()
+        torch.cuda.synchronize()
+        for name, ps, opt, qs, ref in (("graph", pa, oa, pc, oc), ("eager", pb, ob, pd, od)):
+            for i, (p, q) in enumerate(zip(ps, qs)):
+                assert torch.equal(p, q), (name, rep, i, shapes[i])
+                assert torch.equal(opt.state[p]["momentum_buffer"], ref.state[q]["momentum_buffer"]), (name, rep, i)
+
+
+def test_step_under_capture_refuses_tensors_that_moved(env):
+    """Recording a step needs the device pointer tables of an earlier eager step.  When a tensor behind a table has moved
+    (here a gradient re-allocated after the eager steps), the step raises instead of recording a copy out of a host
+    buffer that is gone by the time the graph replays."""
+    dev, mu = env["dev"], env["mu"]
+    g = torch.Generator().manual_seed(9)
+    ps = [torch.nn.Parameter((torch.randn(256, 384, generator=g) * 0.02).to(dev)) for _ in range(3)]
+    for p in ps:
+        p.grad = (torch.randn(p.shape, generator=g) * 0.01).to(dev)
+    opt = mu.Muon([dict(params=ps, use_muon=True, **MUON_HP)])
+    opt.step()
+    opt.step()
+    torch.cuda.synchronize()
+    keep = ps[0].grad  # stays alive, so the clone lands elsewhere
+    ps[0].grad = keep.clone()
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(env["abi"].MuonHipError, match="capture"):
+        with torch.cuda.graph(graph):
+            opt.step()
+    torch.cuda.synchronize()
+    opt.step()  # eager steps go on as before
+    torch.cuda.synchronize()
 
 
 def test_reference_bug_compat_and_rms_scale(env):

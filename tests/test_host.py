@@ -278,12 +278,12 @@ def test_argument_errors_are_reported_before_any_launch():
     rejected(lib.muon_hip_pack_bf16(None, 0, 64, 8, 64, tbl, 256, 64, 1, None), EINVAL, "null tensor")
     rejected(lib.muon_hip_pack_bf16(tbl, 0, 32, 8, 64, tbl, 256, 64, 1, None), ESHAPE, "pack")
     rejected(lib.muon_hip_unpack_bf16(tbl, 256, 48, tbl, 0, 64, 8, 48, 1, None), ESHAPE, "unpack")
-    rejected(lib.muon_hip_syrk_bf16(tbl, tbl, 256, 300, 1, _abi.CFG_AUTO, None), ESHAPE, "multiples")
-    rejected(lib.muon_hip_syrk_bf16(tbl, tbl, 512, 512, 1, 17, None), EINVAL, "unknown GEMM configuration")
-    rejected(lib.muon_hip_syrk_bf16(None, tbl, 512, 512, 1, _abi.CFG_AUTO, None), EINVAL, "null operand")
-    rejected(lib.muon_hip_sympoly_bf16(tbl, tbl, 512, 1, 1.0, 1.0, _abi.CFG_AUTO, None), EINVAL, "aliased")
-    rejected(lib.muon_hip_bx_axpy_bf16(tbl, tbl + 64, tbl + 64, 512, 512, 1, 1.0, _abi.CFG_AUTO, None), EINVAL, "alias")
-    rejected(lib.muon_hip_bx_axpy_bf16(tbl, tbl + 64, tbl + 128, 512, 640, 1, 1.0, _abi.CFG_256_PINGPONG, None),
+    rejected(lib.muon_hip_syrk_bf16(tbl, tbl, 256, 300, 1, _abi.CFG_AUTO, None, None), ESHAPE, "multiples")
+    rejected(lib.muon_hip_syrk_bf16(tbl, tbl, 512, 512, 1, 17, None, None), EINVAL, "unknown GEMM configuration")
+    rejected(lib.muon_hip_syrk_bf16(None, tbl, 512, 512, 1, _abi.CFG_AUTO, None, None), EINVAL, "null operand")
+    rejected(lib.muon_hip_sympoly_bf16(tbl, tbl, 512, 1, 1.0, 1.0, _abi.CFG_AUTO, None, None), EINVAL, "aliased")
+    rejected(lib.muon_hip_bx_axpy_bf16(tbl, tbl + 64, tbl + 64, 512, 512, 1, 1.0, _abi.CFG_AUTO, None, None), EINVAL, "alias")
+    rejected(lib.muon_hip_bx_axpy_bf16(tbl, tbl + 64, tbl + 128, 512, 640, 1, 1.0, _abi.CFG_256_PINGPONG, None, None),
              ESHAPE, "multiples")
     rejected(lib.muon_hip_adamw(None, tbl, tbl, tbl, F32, 4, 1, 1e-3, 0.9, 0.95, 1e-8, 0.0, None), EINVAL, "null tensor")
     rejected(lib.muon_hip_adamw(tbl, tbl, tbl, tbl, F32, 4, 0, 1e-3, 0.9, 0.95, 1e-8, 0.0, None), EINVAL, "step")
@@ -304,18 +304,21 @@ def test_argument_errors_are_reported_before_any_launch():
     rejected(lib.muon_hip_clip_scale(tbl, tbl, tbl, 1, 1, F32, None, F32, 1.0, None), EINVAL, "null total")
     rejected(lib.muon_hip_clip_scale(tbl, tbl, tbl, 1, 1 << 31, F32, tbl, F32, 1.0, None), ESHAPE, "chunks exceed")
     rejected(lib.muon_hip_timing_read(99, None, None), EINVAL, "kernel id")
-    rejected(lib.muon_hip_mfma_probe(None, tbl, 0, 10, None, None), EINVAL, "null buffer")
-    rejected(lib.muon_hip_mfma_probe(tbl, tbl, 2, 10, None, None), EINVAL, "shape")
+    rejected(lib.muon_hip_syrk_bf16(tbl, tbl + 64, 512, 512, 1, _abi.CFG_AUTO, tbl + 8, None), EINVAL, "64-byte aligned")
+    rejected(lib.muon_hip_timing_reserve(-1), EINVAL, "can be reserved")
     rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, (1 << 20) + 1, F32, tbl, None), ESHAPE, "built-in scratch")
     rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, 1, F32, None, None), EINVAL, "null output")
 
 
 def test_chunk_choice_lands_on_whole_rounds():
-    """Matrices per grouped launch: within the workspace cap (plus an eighth), whole rounds of the 256 compute units
-    where the shape allows, never more than the bucket holds, never zero."""
+    """Matrices per grouped launch: never beyond the workspace cap (a hard limit) or the 65535 matrices a library call
+    takes, whole rounds of the 256 compute units where the shape allows, never more than the bucket holds, never zero."""
     pick = muon_utils._pick_chunk
-    assert pick(12288, 248, 768, 2048) == 256  # 6 and 24 tiles per matrix: 6 and 24 whole rounds
+    assert pick(12288, 260, 768, 2048) == 256  # 6 and 24 tiles per matrix: 6 and 24 whole rounds
+    assert pick(12288, 248, 768, 2048) <= 248
+    assert pick(200000, 65535, 37, 53) == 65535 and pick(200000, 1 << 20, 37, 53) == 65535
+    assert pick(200000, 70000, 768, 2048) <= 65535
     assert pick(5, 248, 768, 2048) == 5 and pick(1, 7, 4096, 12288) == 1 and pick(100, 1, 4096, 4096) == 1
     for n, cap, rows, cols in ((72, 15, 4096, 4096), (72, 7, 12288, 4096), (36, 7, 4096, 12288), (24, 91, 896, 4864)):
         nb = pick(n, cap, rows, cols)
-        assert 1 <= nb <= min(n, cap + cap // 8)
+        assert 1 <= nb <= min(n, cap)
