@@ -19,14 +19,20 @@ from .multi_tensor import TensorListTable
 @torch.no_grad()
 def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=False, foreach=None) -> Tensor:
     """Same signature and return value (the total norm, a 0-d tensor on the gradients' device) as
-    fsdp2_clip_grad_norm_.  Only the 2-norm has a kernel; `foreach` is accepted and ignored (every
-    call is one launch per dtype)."""
+    fsdp2_clip_grad_norm_.  norm_type 2 (the default) and inf have kernels, both bit-identical to torch's result in
+    bf16; other orders would need a power function whose roundings differ from torch's and are refused.  `foreach` is
+    accepted and ignored (every call is one launch per dtype)."""
     if isinstance(parameters, Tensor):
         parameters = [parameters]
     else:
         parameters = list(parameters)
-    if float(norm_type) != 2.0:
-        raise NotImplementedError(f"only norm_type=2 has a HIP kernel (got {norm_type})")
+    norm_type = float(norm_type)
+    if norm_type == 2.0:
+        kind = _abi.NORM_L2
+    elif norm_type == float("inf"):
+        kind = _abi.NORM_INF
+    else:
+        raise NotImplementedError(f"norm_type 2 and inf have HIP kernels (got {norm_type})")
     grads = [p.grad for p in parameters if p.grad is not None]
     if len(grads) == 0:
         return torch.tensor(0.0)  # what _get_total_norm returns for an empty list
@@ -35,12 +41,14 @@ def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=Fals
             raise _abi.MuonHipError(f"gradients must live on a GPU: this build has no CPU path (got {g.device})")
     dev = grads[0].device
     groups: "OrderedDict[torch.dtype, list]" = OrderedDict()
+    strided = []  # gradients with other than row-major strides are scaled through a row-major copy that is written back
     for g in grads:
         if g.device != dev:
             raise NotImplementedError("gradients on several devices")
-        groups.setdefault(g.dtype, []).append(g if g.is_contiguous() else None)
-    if any(g is None for gs in groups.values() for g in gs):
-        raise NotImplementedError("gradients must be contiguous")
+        c = g if g.is_contiguous() else g.contiguous()
+        if c is not g:
+            strided.append((g, c))
+        groups.setdefault(g.dtype, []).append(c)
     lib = _abi.lib()
     # torch stacks the per-tensor norms of all dtype groups; stacking promotes, so the total has the widest dtype
     out_dtype = torch.float32 if torch.float32 in groups else torch.bfloat16
@@ -57,16 +65,16 @@ def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=Fals
             if tab.chunks > 0:
                 partials = torch.empty(tab.chunks, dtype=torch.float32, device=dev)
                 _abi.check(lib.muon_hip_grad_norms(tab.role_ptrs[0], tab.numel_ptr, tab.chunk_start_ptr, tab.n, tab.chunks,
-                                                   _abi.dtype_code(dt), partials.data_ptr(), norms.data_ptr() + 4 * off, s),
+                                                   _abi.dtype_code(dt), kind, partials.data_ptr(), norms.data_ptr() + 4 * off, s),
                            "grad_norms")
             else:
                 norms[off:off + tab.n].zero_()
             off += tab.n
-        _abi.check(lib.muon_hip_total_norm(norms.data_ptr(), n_total, _abi.dtype_code(out_dtype), total_f32.data_ptr(),
+        _abi.check(lib.muon_hip_total_norm(norms.data_ptr(), n_total, _abi.dtype_code(out_dtype), kind, total_f32.data_ptr(),
                                            total.data_ptr(), s), "total_norm")
         if error_if_nonfinite and not bool(torch.isfinite(total)):
             raise RuntimeError(
-                f"The total norm of order {float(norm_type)} for gradients from `parameters` is non-finite, so it "
+                f"The total norm of order {norm_type} for gradients from `parameters` is non-finite, so it "
                 "cannot be clipped. To disable this error and scale the gradients by the non-finite norm anyway, "
                 "set `error_if_nonfinite=False`")
         for dt, tab in tables:
@@ -74,6 +82,8 @@ def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=Fals
                 _abi.check(lib.muon_hip_clip_scale(tab.role_ptrs[0], tab.numel_ptr, tab.chunk_start_ptr, tab.n, tab.chunks,
                                                    _abi.dtype_code(dt), total_f32.data_ptr(), _abi.dtype_code(out_dtype),
                                                    float(max_norm), s), "clip_scale")
+        for g, c in strided:
+            g.copy_(c)
     return total
 
 

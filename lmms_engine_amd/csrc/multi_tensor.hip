@@ -2,9 +2,10 @@
 //
 //   adamw_multi      : adam_update + the Adam branch of step_fsdp (muon_utils.py:178-183,
 //                      :468-477) for every tensor of a parameter group
-//   sqnorm / norms   : the 2-norm torch's _get_total_norm computes for
+//   sqnorm / norms   : the norm torch's _get_total_norm computes for
 //                      fsdp2_clip_grad_norm_ (utils/fsdp2_utils.py:234-255): per-tensor norms
-//                      rounded to the tensor dtype, then the norm of those norms
+//                      rounded to the tensor dtype, then the norm of those norms; the 2-norm, or the
+//                      infinity norm (largest magnitude, a NaN anywhere makes the result NaN, as torch's max does)
 //   clip_scale_multi : _clip_grads_with_norm_: g *= clamp(max_norm / (total + 1e-6), max=1)
 //
 // A tensor list is cut into chunks of MUON_MULTI_CHUNK elements; chunk_start[t] is the index of
@@ -146,7 +147,21 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
     return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-template <typename T>
+// Largest of two magnitudes; a NaN on either side wins (fmaxf would drop it).
+__device__ __forceinline__ float nan_max(float a, float b) { return (a != a) ? a : (b != b) ? b : fmaxf(a, b); }
+
+__device__ __forceinline__ float block_max_256(float v, float* red) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = nan_max(v, __shfl_xor(v, off, 64));
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    return nan_max(nan_max(red[0], red[1]), nan_max(red[2], red[3]));
+}
+
+// INF = false: sum of squares of a chunk; true: its largest magnitude.
+template <typename T, bool INF>
 __global__ void __launch_bounds__(256)
 sqnorm_multi_kernel(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, float* partials) {
     __shared__ float red[4];
@@ -159,37 +174,39 @@ sqnorm_multi_kernel(const void* const* g_ptrs, const long* numel, const long* ch
         float v[8];
         Mt<T>::load8(g + i * 8, v);
 #pragma unroll
-        for (int k = 0; k < 8; ++k) ss = fmaf(v[k], v[k], ss);
+        for (int k = 0; k < 8; ++k) ss = INF ? nan_max(ss, fabsf(v[k])) : fmaf(v[k], v[k], ss);
     }
     for (long i = n8 * 8 + threadIdx.x; i < r.len; i += 256) {
         const float v = Mt<T>::load(g + i);
-        ss = fmaf(v, v, ss);
+        ss = INF ? nan_max(ss, fabsf(v)) : fmaf(v, v, ss);
     }
-    ss = block_sum_256(ss, red);
+    ss = INF ? block_max_256(ss, red) : block_sum_256(ss, red);
     if (threadIdx.x == 0) partials[blockIdx.x] = ss;
 }
 
-// One block per tensor: its partial sums in a fixed order -> norm, rounded to the tensor dtype.
+// One block per tensor: its partial results in a fixed order -> norm, rounded to the tensor dtype.
+template <bool INF>
 __global__ void __launch_bounds__(256)
 tensor_norm_kernel(const float* partials, const long* chunk_start, int dtype, float* norms) {
     __shared__ float red[4];
     const int t = blockIdx.x;
     float ss = 0.f;
-    for (long c = chunk_start[t] + threadIdx.x; c < chunk_start[t + 1]; c += 256) ss += partials[c];
-    ss = block_sum_256(ss, red);
-    if (threadIdx.x == 0) norms[t] = rnd_dtype(sqrtf(ss), dtype);
+    for (long c = chunk_start[t] + threadIdx.x; c < chunk_start[t + 1]; c += 256) ss = INF ? nan_max(ss, partials[c]) : ss + partials[c];
+    ss = INF ? block_max_256(ss, red) : block_sum_256(ss, red);
+    if (threadIdx.x == 0) norms[t] = INF ? ss : rnd_dtype(sqrtf(ss), dtype);
 }
 
 // One block: norm of the per-tensor norms, rounded to the result dtype; written as fp32 (for the
 // scaling kernel) and in the result dtype (the tensor the caller returns).
+template <bool INF>
 __global__ void __launch_bounds__(256)
 total_norm_kernel(const float* norms, int n, int dtype, float* total_f32, void* total_typed) {
     __shared__ float red[4];
     float ss = 0.f;
-    for (int t = threadIdx.x; t < n; t += 256) ss = fmaf(norms[t], norms[t], ss);
-    ss = block_sum_256(ss, red);
+    for (int t = threadIdx.x; t < n; t += 256) ss = INF ? nan_max(ss, norms[t]) : fmaf(norms[t], norms[t], ss);
+    ss = INF ? block_max_256(ss, red) : block_sum_256(ss, red);
     if (threadIdx.x == 0) {
-        const float tn = rnd_dtype(sqrtf(ss), dtype);
+        const float tn = INF ? ss : rnd_dtype(sqrtf(ss), dtype);
         *total_f32 = tn;
         if (dtype == MUON_HIP_BF16) *(bf16_t*)total_typed = f2bf(tn);
         else *(float*)total_typed = tn;
@@ -253,23 +270,25 @@ hipError_t launch_adamw_multi(const MultiTensorList& l, const void* const* g_ptr
     return hipGetLastError();
 }
 
-hipError_t launch_tensor_norms(const MultiTensorList& l, int dtype, float* partials, float* norms, hipStream_t stream) {
+hipError_t launch_tensor_norms(const MultiTensorList& l, int dtype, bool inf_norm, float* partials, float* norms,
+                               hipStream_t stream) {
     dim3 grid((unsigned)l.chunks), block(256);
-    if (dtype == MUON_HIP_F32)
-        hipLaunchKernelGGL((sqnorm_multi_kernel<float>), grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n, partials);
-    else if (dtype == MUON_HIP_BF16)
-        hipLaunchKernelGGL((sqnorm_multi_kernel<bf16_t>), grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n, partials);
-    else
-        return hipErrorInvalidValue;
+    if (dtype != MUON_HIP_F32 && dtype != MUON_HIP_BF16) return hipErrorInvalidValue;
+    const bool f32 = dtype == MUON_HIP_F32;
+    auto k = f32 ? (inf_norm ? sqnorm_multi_kernel<float, true> : sqnorm_multi_kernel<float, false>)
+                 : (inf_norm ? sqnorm_multi_kernel<bf16_t, true> : sqnorm_multi_kernel<bf16_t, false>);
+    hipLaunchKernelGGL(k, grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n, partials);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(tensor_norm_kernel, dim3((unsigned)l.n), block, 0, stream, partials, l.chunk_start, dtype, norms);
+    auto k2 = inf_norm ? tensor_norm_kernel<true> : tensor_norm_kernel<false>;
+    hipLaunchKernelGGL(k2, dim3((unsigned)l.n), block, 0, stream, partials, l.chunk_start, dtype, norms);
     return hipGetLastError();
 }
 
-hipError_t launch_total_norm(const float* norms, int n, int dtype, float* total_f32, void* total_typed,
+hipError_t launch_total_norm(const float* norms, int n, int dtype, bool inf_norm, float* total_f32, void* total_typed,
                              hipStream_t stream) {
-    hipLaunchKernelGGL(total_norm_kernel, dim3(1), dim3(256), 0, stream, norms, n, dtype, total_f32, total_typed);
+    auto k = inf_norm ? total_norm_kernel<true> : total_norm_kernel<false>;
+    hipLaunchKernelGGL(k, dim3(1), dim3(256), 0, stream, norms, n, dtype, total_f32, total_typed);
     return hipGetLastError();
 }
 

@@ -501,17 +501,18 @@ class Muon(torch.optim.Optimizer):
             if group["use_muon"]:
                 for p in group["params"]:
                     _require_cuda(p, "a Muon parameter")
-                    if not p.is_contiguous():
-                        raise NotImplementedError("Muon parameters must be contiguous")
                     u = p.grad.reshape(p.shape)
                     u = u if u.is_contiguous() else u.contiguous()
+                    pc = p if p.is_contiguous() else p.detach().contiguous()  # row-major copy, written back below
                     with torch.cuda.device(p.device):
                         _abi.check(
-                            lib.muon_hip_decay_update(p.data_ptr(), _abi.dtype_code(p.dtype), u.data_ptr(),
+                            lib.muon_hip_decay_update(pc.data_ptr(), _abi.dtype_code(p.dtype), u.data_ptr(),
                                                       _abi.dtype_code(u.dtype), p.numel(), float(group["lr"]),
                                                       float(group["weight_decay"]), _abi.stream_ptr(p.device)),
                             "decay_update",
                         )
+                    if pc is not p:
+                        p.copy_(pc)
             else:
                 self._adam_group_step(group)
         return loss
@@ -564,6 +565,7 @@ class Muon(torch.optim.Optimizer):
         for group in self.param_groups:
             if group["use_muon"]:
                 buckets: "OrderedDict[tuple, list]" = OrderedDict()
+                strided = []
                 for i, p in enumerate(group["params"]):
                     assert p.ndim == 2, p.shape
                     if p.grad is None:
@@ -578,12 +580,16 @@ class Muon(torch.optim.Optimizer):
                             dq.popleft().finish()
                         continue
                     _require_cuda(p, "a Muon parameter")
-                    if not p.is_contiguous():
-                        raise NotImplementedError("Muon parameters must be contiguous")
+                    # The kernels read row-major tensors.  A parameter, gradient or momentum buffer with other strides
+                    # (the reference's torch expressions take any) steps through row-major copies that are written back.
                     g = p.grad if p.grad.is_contiguous() else p.grad.contiguous()
                     m = state["momentum_buffer"]
+                    pc = p if p.is_contiguous() else p.detach().contiguous()
+                    mc = m if m.is_contiguous() else m.contiguous()
+                    if pc is not p or mc is not m or (g is not p.grad and self.write_back_grad):
+                        strided.append((p, pc, m, mc, g))
                     key = (p.device, tuple(p.shape), p.dtype, g.dtype, m.dtype)
-                    buckets.setdefault(key, []).append((p, g, m))
+                    buckets.setdefault(key, []).append((pc, g, mc))
                 ns_steps, nesterov = group["ns_steps"], group["nesterov"]
                 if self.reference_bug_compat:
                     ns_steps, nesterov = int(bool(group["nesterov"])), bool(group["ns_steps"])
@@ -591,6 +597,13 @@ class Muon(torch.optim.Optimizer):
                     ps, gs, ms = (list(t) for t in zip(*items))
                     _muon_bucket_step(ps, gs, ms, group, ns_steps, nesterov, self.write_back_grad, self._workspaces,
                                       self.workspace_limit_bytes, self._pointer_tables)
+                for p, pc, m, mc, g in strided:
+                    if pc is not p:
+                        p.copy_(pc)
+                    if mc is not m:
+                        m.copy_(mc)
+                    if g is not p.grad and self.write_back_grad:
+                        p.grad.copy_(g)
             else:
                 self._adam_group_step(group)
 
@@ -609,10 +622,9 @@ def _adamw_group(items, group: dict) -> None:
     from .multi_tensor import TensorListTable
 
     buckets: "OrderedDict[tuple, list]" = OrderedDict()
+    strided = []  # tensors with other than row-major strides step through row-major copies that are written back
     for p, grad, e1, e2, step in items:
         _require_cuda(p, "an AdamW parameter")
-        if not (p.is_contiguous() and e1.is_contiguous() and e2.is_contiguous()):
-            raise NotImplementedError("AdamW-fallback parameters and state must be contiguous")
         if e1.dtype != p.dtype or e2.dtype != p.dtype:
             raise NotImplementedError("AdamW-fallback state must have the parameter's dtype")
         if p.numel() == 0:
@@ -620,6 +632,10 @@ def _adamw_group(items, group: dict) -> None:
         g = grad
         if g.dtype != p.dtype or not g.is_contiguous():
             g = g.to(p.dtype).contiguous()
+        if not (p.is_contiguous() and e1.is_contiguous() and e2.is_contiguous()):
+            pairs = [(t, t if t.is_contiguous() else t.detach().contiguous()) for t in (p, e1, e2)]
+            strided.extend(pr for pr in pairs if pr[0] is not pr[1])
+            p, e1, e2 = (c for _, c in pairs)
         buckets.setdefault((p.device, p.dtype), []).append((p, g, e1, e2, step))
     b1, b2 = float(group["betas"][0]), float(group["betas"][1])
     for (dev, dt), its in buckets.items():
@@ -634,6 +650,8 @@ def _adamw_group(items, group: dict) -> None:
                 ),
                 "adamw_multi",
             )
+    for t, c in strided:
+        t.copy_(c)
 
 
 def _adamw_tensor(p: Tensor, grad: Tensor, exp_avg: Tensor, exp_avg_sq: Tensor, step: int, group: dict) -> None:

@@ -136,11 +136,58 @@ def test_clip_grad_norm_edge_cases(env):
     assert torch.isinf(out) and torch.isnan(p.grad).all()
     with pytest.raises(NotImplementedError):
         clip.clip_grad_norm_([p], 1.0, norm_type=1.0)
+    p.grad = torch.tensor([1.0, float("nan"), 3.0] + [0.0] * 7, device=dev)
+    assert torch.isnan(clip.clip_grad_norm_([p], 1.0, norm_type=float("inf")))  # a NaN is the largest, as in torch.max
     q = torch.nn.Parameter(torch.zeros(4))
     q.grad = torch.ones(4)
     with pytest.raises(env["abi"].MuonHipError):
         clip.clip_grad_norm_([q], 1.0)  # CPU gradients: no fallback
     assert clip.fsdp2_clip_grad_norm_ is clip.clip_grad_norm_
+
+
+@pytest.mark.parametrize("dtypes", [(torch.float32,), (torch.bfloat16,), (torch.float32, torch.bfloat16)])
+def test_clip_grad_norm_infinity_norm_and_strided_gradients(env, dtypes):
+    """norm_type=inf (fsdp2_clip_grad_norm_ forwards any norm_type to torch, utils/fsdp2_utils.py:244-254): the largest
+    magnitude over all gradients, exact in any order, so the total and the scaled gradients must equal torch's on the
+    CPU (fp32 gradients to 1e-6: the coefficient's reciprocal).  Gradients that are transposed or sliced views step
+    through a row-major copy and are written back in place."""
+    clip, dev = env["clip"], env["dev"]
+    gen = torch.Generator().manual_seed(41)
+    shapes = [(300, 70), (16384 * 2 + 5,), (9,), (64, 33)]
+    ps, cpu = [], []
+    for i, s in enumerate(shapes):
+        dt = dtypes[i % len(dtypes)]
+        g = (2.5 * torch.randn(*s, generator=gen)).to(dt)
+        if i == 0:   # a transposed view: dense, not row-major
+            gd, gc = g.to(dev).t().contiguous().t(), g.clone()
+        elif i == 3:  # a column slice: strided with gaps
+            wide_d, wide_c = torch.zeros(64, 66, dtype=dt, device=dev), torch.zeros(64, 66, dtype=dt)
+            gd, gc = wide_d[:, ::2], wide_c[:, ::2]
+            gd.copy_(g.to(dev))
+            gc.copy_(g)
+        else:
+            gd, gc = g.to(dev), g.clone()
+        assert (i in (0, 3)) == (not gd.is_contiguous())
+        p, c = torch.nn.Parameter(torch.zeros(*s, dtype=dt, device=dev)), torch.nn.Parameter(torch.zeros(*s, dtype=dt))
+        p.grad, c.grad = gd, gc
+        ps.append(p)
+        cpu.append(c)
+    for it, (norm_type, max_norm) in enumerate(((float("inf"), 1.0), (2.0, 0.5), (float("inf"), 100.0))):
+        got = clip.clip_grad_norm_(ps, max_norm, norm_type=norm_type)
+        ref = torch.nn.utils.clip_grad_norm_(cpu, max_norm, norm_type=norm_type, foreach=False)
+        torch.cuda.synchronize()
+        assert got.dtype == ref.dtype
+        # exact while both sides hold the same gradients: always in bf16, in fp32 until the first scaling
+        if got.dtype == torch.bfloat16 or it == 0:
+            assert got.item() == ref.item(), (norm_type, got.item(), ref.item())
+        else:
+            assert abs(got.item() - ref.item()) <= 1e-6 * ref.item()
+        for i, (p, c) in enumerate(zip(ps, cpu)):
+            assert (i in (0, 3)) == (not p.grad.is_contiguous())  # scaled in place: the views are still views
+            if p.grad.dtype == torch.float32:
+                assert rel_fro(p.grad, c.grad) <= 1e-6
+            else:
+                assert torch.equal(p.grad.cpu(), c.grad)
 
 
 def test_clip_grad_norm_full_size(env):

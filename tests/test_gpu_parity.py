@@ -977,6 +977,45 @@ def test_step_under_capture_refuses_tensors_that_moved(env):
     torch.cuda.synchronize()
 
 
+def test_strided_parameters_and_state_step_like_row_major_ones(env):
+    """The reference's torch expressions take parameters of any strides (muon_utils.py:324-325, :476-477).  A Muon
+    parameter that is a transposed view (its momentum buffer, made by zeros_like, then has the same strides), a
+    parameter with a strided gradient, and an AdamW parameter that is a transposed view step through row-major copies:
+    values must equal those of row-major twins bit for bit over two steps, and the strides must survive."""
+    mu, dev = env["mu"], env["dev"]
+    gen = torch.Generator().manual_seed(61)
+    w = [0.02 * torch.randn(256, 384, generator=gen), 0.02 * torch.randn(384, 256, generator=gen), 0.02 * torch.randn(96, 40, generator=gen)]
+    e = torch.randn(50, 30, generator=gen)
+
+    def as_t_view(t):  # same values, column-major storage
+        return t.to(dev).t().contiguous().t()
+
+    pa = [torch.nn.Parameter(w[0].to(dev)), torch.nn.Parameter(w[1].to(dev)), torch.nn.Parameter(w[2].to(dev))]
+    pb = [torch.nn.Parameter(as_t_view(w[0])), torch.nn.Parameter(w[1].to(dev)), torch.nn.Parameter(as_t_view(w[2]))]
+    ea, eb = torch.nn.Parameter(e.to(dev)), torch.nn.Parameter(as_t_view(e))
+    assert not pb[0].is_contiguous() and not eb.is_contiguous()
+    ahp = dict(lr=1e-3, betas=(0.9, 0.95), eps=1e-10, weight_decay=0.01)
+    oa = mu.Muon([dict(params=list(pa), use_muon=True, **MUON_HP), dict(params=[ea], use_muon=False, **ahp)], write_back_grad=True)
+    ob = mu.Muon([dict(params=list(pb), use_muon=True, **MUON_HP), dict(params=[eb], use_muon=False, **ahp)], write_back_grad=True)
+    for step in range(2):
+        gs = [1e-3 * torch.randn(*t.shape, generator=gen) for t in w]
+        ge = torch.randn(50, 30, generator=gen)
+        for p, q, g in zip(pa, pb, gs):
+            p.grad = g.to(dev)
+            q.grad = as_t_view(g) if q is not pb[0] else g.to(dev)  # strided gradients for the row-major and one strided parameter
+        ea.grad, eb.grad = ge.to(dev), as_t_view(ge)
+        oa.step()
+        ob.step()
+        torch.cuda.synchronize()
+        for p, q in zip(pa + [ea], pb + [eb]):
+            assert torch.equal(p.detach(), q.detach()), (step, tuple(p.shape))
+        for p, q in zip(pa, pb):
+            assert torch.equal(oa.state[p]["momentum_buffer"], ob.state[q]["momentum_buffer"])
+            assert torch.equal(p.grad, q.grad)  # write_back_grad: the blend reaches a strided gradient too
+        assert torch.equal(oa.state[ea]["exp_avg_sq"], ob.state[eb]["exp_avg_sq"])
+    assert pb[0].stride() == (1, 256) and ob.state[pb[0]]["momentum_buffer"].stride() == (1, 256) and eb.stride() == (1, 50)
+
+
 def test_reference_bug_compat_and_rms_scale(env):
     """The reference's single-device call site runs range(True) = 1 NS iteration; the flag reproduces it."""
     mu, O = env["mu"], env["O"]
