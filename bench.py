@@ -183,6 +183,25 @@ def extras(params, pd, dev, reps):
     return res
 
 
+def hbm_reference(dev, gib=2, reps=10):
+    """What torch's own streaming kernels reach on this box, as bytes moved per second: a read-only reduction, an
+    in-place multiply (one read and one write per element, the mix of the momentum kernel) and a copy (the mix of the
+    normalisation).  The elementwise kernels of the step are to be read against these as well as against the 8 TB/s."""
+    import torch
+
+    n = gib << 28  # fp32 elements
+    a = torch.empty(n, dtype=torch.float32, device=dev).normal_()
+    b = torch.empty_like(a)
+    nbytes = 4.0 * n
+    res = {}
+    for name, fn, moved in (("read_only_norm", lambda: torch.linalg.vector_norm(a), nbytes), ("in_place_multiply", lambda: a.mul_(1.0000001), 2 * nbytes),
+                            ("copy", lambda: b.copy_(a), 2 * nbytes)):
+        ms = _event_ms(fn, reps, torch, warm=2)
+        res[name] = dict(gbs=moved / (ms * 1e-3) / 1e9, frac_hbm_peak=moved / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS)
+    res["what"] = f"torch kernels over {gib} GiB fp32 buffers, {reps} calls each"
+    return res
+
+
 def _event_ms(fn, reps, torch, warm=1):
     """Mean milliseconds of fn() over `reps` calls after `warm` warm-up calls, from events on the current stream."""
     for _ in range(warm):
@@ -352,6 +371,8 @@ def main():
     ap.add_argument("--extras", action="store_true",
                     help="also time the two neighbours of the Muon step, outside the timed region: gradient-norm clipping "
                          "over the same gradients and the AdamW fallback over an embedding + lm_head + norm-vector group")
+    ap.add_argument("--no-hbm-reference", action="store_true",
+                    help="skip the streaming rates of torch's own kernels on this box (after the timed region)")
     ap.add_argument("--no-gpu-oracle", action="store_true",
                     help="skip the second baseline (the reference's expressions unfused in torch on this GPU, and the "
                          "library bf16 GEMM on the shapes of the dominant kernel), which runs after the timed region")
@@ -524,6 +545,8 @@ def main():
     if args.operand_power:
         out["operand_power"] = operand_power(dev)
         out["mfma_probe"] = mfma_probe(dev)
+    if not args.no_hbm_reference:
+        out["hbm_reference"] = hbm_reference(dev)
     if not args.no_gpu_oracle:
         moms = [opt.state[p]["momentum_buffer"] for p in params]
         out["gpu_oracle"] = gpu_oracle(params, moms, shapes, flops_step)

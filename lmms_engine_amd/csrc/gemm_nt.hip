@@ -1,7 +1,7 @@
 // GEMM family for the Newton-Schulz chain on gfx950, built on v_mfma_f32_16x16x32_bf16.
 //
 // Why the 16x16x32 instruction: under matrix-pipe load the part lowers its clock to stay inside its power
-// limit, and on operands with random mantissas a loop of nothing but MFMAs (muon_hip_mfma_probe) sustains about
+// limit, and on operands with random mantissas a loop of nothing but MFMAs (probe.hip, a measurement library of its own) sustains about
 // 1.85 PFLOP/s with 32x32x16 and about 2.09 with 16x16x32 (both reach 2.45 on constant operands): the deeper dot
 // product updates each fp32 accumulator half as often per FLOP.  The same kernels built on 32x32x16 ran 4 to 8 %
 // slower at a 3 to 9 % lower clock.  Operand fragment: lane l holds row l%16, eight consecutive k from 8*(l/16)
@@ -1032,7 +1032,7 @@ __global__ void __launch_bounds__(WGM* WGN * 64) gemm_nt_pp_kernel(const GemmArg
     pp_tile<BM, BN, WGM, WGN, EPI>(g, decode_tile<EPI>(g), smem);
 }
 
-// The same with a split tail: when the tile count leaves the last round of the 256 CUs mostly empty,
+// The same with a split tail: when the tile count leaves the last round of the compute units mostly empty,
 // the first g.big_blocks workgroups compute 256x256 tiles as above and every remaining tile is cut
 // into four 128x128 tiles, one workgroup each, which fill the CUs that would otherwise idle for a
 // whole tile time.  The lower-left quarter of a diagonal tile of the symmetric kernels is the mirror

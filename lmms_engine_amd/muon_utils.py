@@ -437,6 +437,7 @@ class Muon(torch.optim.Optimizer):
         self.keep_workspace = bool(keep_workspace)
         self._workspaces = {}
         self._pointer_tables = {}  # per bucket chunk: (pointers, device table) of the last step
+        self._recorded = False     # a step has been recorded into a HIP graph: workspace and tables must stay
         if not reference_bug_compat and not is_deepspeed_enabled:
             _note_keyword_semantics()
         for group in param_groups:
@@ -519,8 +520,17 @@ class Muon(torch.optim.Optimizer):
 
     def release_workspace(self) -> None:
         """Drop the Newton-Schulz workspace (it is re-allocated by the next step): for callers that want the
-        memory back between optimizer steps, e.g. for activations."""
+        memory back between optimizer steps, e.g. for activations.  A HIP graph recorded from step() holds the
+        workspace's address, so after a recording the workspace stays until `forget_recordings()` says that no such
+        graph will be replayed any more."""
+        if self._recorded:
+            raise RuntimeError("a recorded HIP graph replays into this workspace: call forget_recordings() once the "
+                               "graph is gone, then release_workspace()")
         self._workspaces.clear()
+
+    def forget_recordings(self) -> None:
+        """Declare that no HIP graph recorded from step() will be replayed again."""
+        self._recorded = False
 
     def _adam_group_step(self, group) -> None:
         items = []
@@ -562,6 +572,10 @@ class Muon(torch.optim.Optimizer):
             with torch.enable_grad():
                 loss = closure()
         dq: deque[Work] = deque()
+        if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+            if not self.keep_workspace:
+                raise RuntimeError("recording a step into a HIP graph needs keep_workspace=True: replays use the workspace")
+            self._recorded = True
         for group in self.param_groups:
             if group["use_muon"]:
                 buckets: "OrderedDict[tuple, list]" = OrderedDict()

@@ -908,6 +908,17 @@ def test_muon_step_replays_from_a_hip_graph(env):
         for i, (p, q) in enumerate(zip(pa, pb)):
             assert torch.equal(p, q), (rep, i, shapes[i])
             assert torch.equal(oa.state[p]["momentum_buffer"], ob.state[q]["momentum_buffer"]), (rep, i)
+    # the recording replays into the optimizer's workspace: it cannot be released while the graph may run again
+    with pytest.raises(RuntimeError, match="recorded"):
+        oa.release_workspace()
+    del graph
+    oa.forget_recordings()
+    oa.release_workspace()
+    ob.release_workspace()
+    oa.step()  # and the next eager step allocates it again
+    ob.step()
+    torch.cuda.synchronize()
+    assert all(torch.equal(p, q) for p, q in zip(pa, pb))
 
 
 def test_two_optimizers_on_two_streams_one_replaying_a_graph(env):
