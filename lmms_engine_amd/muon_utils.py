@@ -77,12 +77,12 @@ def _workspace(nbytes: int, device) -> Tensor:
 
 
 def _pointer_table(tensors, device, cache=None, key=None) -> Tensor:
-    """Device table of the tensors' base pointers.  With a cache, a table whose pointers have not changed since the last
-    call under `key` is handed back as it is: no host allocation and no copy, which is what lets a step over static
-    tensors be recorded into a HIP graph (and saves the copy otherwise)."""
+    """Device table of the tensors' base pointers.  With a cache (a _TableCache), a table whose pointers have not changed
+    since the last call under `key` is handed back as it is: no host allocation and no copy, which is what lets a step
+    over static tensors be recorded into a HIP graph (and saves the copy otherwise)."""
     ptrs = tuple(t.data_ptr() for t in tensors)
     if cache is not None:
-        hit = cache.get(key)
+        hit = cache.tables.get(key)
         if hit is not None and hit[0] == ptrs and hit[1].device == device:
             return hit[1]
     if torch.cuda.is_current_stream_capturing():
@@ -96,14 +96,29 @@ def _pointer_table(tensors, device, cache=None, key=None) -> Tensor:
     host = torch.tensor(ptrs, dtype=torch.int64, pin_memory=True)
     table = host.to(device, non_blocking=True)
     if cache is not None:
-        old = cache.get(key)
-        if old is not None:
-            # a graph recorded earlier may still read the old table: keep it alive instead of handing its memory
-            # back to the allocator (bounded: one generation per change of addresses)
-            cache.setdefault("_retired", []).append(old[1])
-            del cache["_retired"][:-64]
-        cache[key] = (ptrs, table)
+        cache.replace(key, ptrs, table)
     return table
+
+
+class _TableCache:
+    """Pointer tables of the last step, per bucket chunk.  A table that a later step replaces is kept alive for a while
+    instead of going back to the allocator: a HIP graph recorded earlier may still read it."""
+
+    KEEP = 64  # replaced tables kept alive (a few KB each)
+
+    def __init__(self):
+        self.tables = {}   # key -> (pointers, device table)
+        self.retired = []
+
+    def __len__(self):
+        return len(self.tables)
+
+    def replace(self, key, ptrs, table) -> None:
+        old = self.tables.get(key)
+        if old is not None:
+            self.retired.append(old[1])
+            del self.retired[:-self.KEEP]
+        self.tables[key] = (ptrs, table)
 
 
 def scale_factor(rows: int, cols: int, rms_scale: bool) -> float:
@@ -436,7 +451,7 @@ class Muon(torch.optim.Optimizer):
         self.workspace_limit_bytes = int(workspace_limit_bytes)
         self.keep_workspace = bool(keep_workspace)
         self._workspaces = {}
-        self._pointer_tables = {}  # per bucket chunk: (pointers, device table) of the last step
+        self._pointer_tables = _TableCache()  # per bucket chunk: the device pointer table of the last step
         self._recorded = False     # a step has been recorded into a HIP graph: workspace and tables must stay
         if not reference_bug_compat and not is_deepspeed_enabled:
             _note_keyword_semantics()

@@ -706,7 +706,7 @@ def test_chunked_bucket_equals_the_unchunked_twin_bitwise(env, rows, cols, n, ca
             opt.step()
         torch.cuda.synchronize()
         (pa, oa), (pb, ob) = twins
-        assert len(oa._pointer_tables) - ("_retired" in oa._pointer_tables) == nchunks
+        assert len(oa._pointer_tables) == nchunks
         assert oa._workspaces[dev].numel() <= limit < ob._workspaces[dev].numel()
         for i in range(n):
             assert torch.equal(pa[i].detach(), pb[i].detach()), f"step {step}, matrix {i}: parameter"
