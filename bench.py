@@ -354,6 +354,40 @@ def mfma_probe(dev, iters=40000, reps=25):
     return res
 
 
+def stream_probe(dev, gib=2, reps=4):
+    """Streaming rate of plain kernels (muon_probe_stream of libmuon_probe.so) against the number of XCDs that take part:
+    a read, a read and a write in place, a copy.  One XCD alone and all eight together bound what the elementwise kernels
+    of the step can reach on this box."""
+    import ctypes
+
+    import torch
+
+    from lmms_engine_amd import _abi
+    from lmms_engine_amd.build import PROBE_LIB
+
+    lib = ctypes.CDLL(PROBE_LIB)
+    lib.muon_probe_stream.restype = ctypes.c_int
+    lib.muon_probe_stream.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_long, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                      ctypes.c_void_p]
+    nbytes = gib << 30
+    a = torch.zeros(nbytes // 4, dtype=torch.float32, device=dev)
+    b = torch.zeros_like(a)
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    res = {}
+    for mode, name in ((0, "read_only"), (1, "in_place"), (2, "copy")):
+        res[name] = {}
+        for nx in (1, 2, 4, 8):
+            def fn():
+                rc = lib.muon_probe_stream(a.data_ptr(), b.data_ptr(), nbytes, mode, nx, sink.data_ptr(), _abi.stream_ptr(dev))
+                assert rc == 0, f"muon_probe_stream failed ({rc})"
+
+            ms = _event_ms(fn, reps, torch, warm=2)
+            moved = nbytes * (1 if mode == 0 else 2)
+            res[name][f"{nx}_xcds"] = dict(gbs=moved / (ms * 1e-3) / 1e9, frac_hbm_peak=moved / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS)
+    res["what"] = f"{gib} GiB buffers, fp32x4 accesses, {reps} launches per point; workgroup b runs on XCD b % 8"
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -380,6 +414,8 @@ def main():
                     help="also time the three product entry points on random and on constant operands of one size")
     ap.add_argument("--operand-power-only", action="store_true",
                     help="run only the --operand-power measurement (for counter runs)")
+    ap.add_argument("--stream-probe-only", action="store_true",
+                    help="run only the streaming-rate measurement against the number of active XCDs")
     ap.add_argument("--gemm-config", type=int, default=-1,
                     help="force one GEMM tile configuration (MUON_HIP_CFG_*; -1 = chosen per kernel and shape)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -406,6 +442,9 @@ def main():
         _abi.check(_abi.lib().muon_hip_set_gemm_config(args.gemm_config), "set_gemm_config")
     if args.operand_power_only:
         print(json.dumps({"operand_power": operand_power(dev), "mfma_probe": mfma_probe(dev)}))
+        return
+    if args.stream_probe_only:
+        print(json.dumps({"stream_probe": stream_probe(dev)}))
         return
     w = WORKLOADS[args.workload]
     layers = args.layers or w["layers"]

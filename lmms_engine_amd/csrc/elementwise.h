@@ -3,7 +3,8 @@
 #include <hip/hip_runtime.h>
 #include "common.h"
 
-#define MUON_MAX_PARTS 4096  // Frobenius partial sums per matrix, at most
+#define MUON_PART_ELEMS 4096   // elements per Frobenius partial sum = per workgroup of the momentum kernel
+#define MUON_MAX_PARTS 65536   // partial sums per matrix, at most (larger matrices put more elements into each)
 
 int momentum_parts(long n);
 hipError_t launch_momentum_norm(const void* const* g_ptrs, const void* const* m_ptrs, int g_dtype, int m_dtype,

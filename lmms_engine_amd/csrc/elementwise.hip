@@ -104,7 +104,11 @@ momentum_norm_kernel(const void* const* g_ptrs, const void* const* m_ptrs, bf16_
     const long n8 = vec ? n / 8 : 0;
     // Each block owns one contiguous run of the matrix (so the blocks resident at any time
     // stream neighbouring DRAM pages); two 8-element groups per thread and trip, all loads
-    // issued before the arithmetic.
+    // issued before the arithmetic.  The launcher sizes the grid for one trip per block (4096 elements): measured on
+    // every bucket of the benchmark sets, many short-lived blocks stream 3 to 5 % faster than blocks that loop four
+    // times, and 11 % faster than the fourteen trips a single 28672 x 8192 matrix used to take under the old cap of
+    // 4096 blocks per matrix (a plain in-place kernel shows the same: 5.98 TB/s at one 16-byte access per thread, 5.52 at
+    // four, 4.27 at eight).
     const long per_block = ((n8 + gridDim.x - 1) / gridDim.x + 511) / 512 * 512;
     const long lo8 = (long)blockIdx.x * per_block, hi8 = lo8 + per_block < n8 ? lo8 + per_block : n8;
     for (long i8 = lo8 + threadIdx.x; i8 < hi8; i8 += 512) {
@@ -197,8 +201,17 @@ __global__ void __launch_bounds__(256) frob_finalize_kernel(const float* partial
     const int b = blockIdx.x;
     if (b == 0 && clear)
         for (int i = threadIdx.x; i < clear_words; i += 256) clear[i] = 0u;
+    // eight partial sums in flight per thread (a matrix of 2^28 elements has 65536 of them), added in a fixed order
+    const float* p = partials + (long)b * nparts;
     float s = 0.f;
-    for (int i = threadIdx.x; i < nparts; i += 256) s += partials[(long)b * nparts + i];
+    int i = threadIdx.x;
+    for (; i + 7 * 256 < nparts; i += 8 * 256) {
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = p[i + k * 256];
+        s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+    }
+    for (; i < nparts; i += 256) s += p[i];
     s = block_sum_256(s, red);
     if (threadIdx.x == 0) {
         const float nrm = rbf(sqrtf(s));
@@ -206,53 +219,78 @@ __global__ void __launch_bounds__(256) frob_finalize_kernel(const float* partial
     }
 }
 
-// One 64x128 tile of the bf16 blend u (parameter layout, rows x cols) divided by d, written into the
-// blocked X (M x K, zero padded to Mp x Kp): directly when the parameter has X's orientation
-// (16 rows of a block back to back = 1 KB runs), through an LDS transpose when rows > cols (X = u^T,
-// 32 rows of a block = 2 KB runs).
+// The bf16 blend u (parameter layout, rows x cols) divided by d, written into the blocked X (M x K, zero padded to
+// Mp x Kp).  Both kernels give a thread as little as one 16-byte load and one 16-byte store: measured on every bucket of
+// the benchmark sets, tiles of 16 x 128 stream 8 % faster than the 64 x 128 tiles (four accesses each way per thread)
+// they replace (5.7 to 5.8 against 5.3 TB/s), the same way a plain in-place kernel loses 8 % from one to four accesses.
+//
+// A parameter in X's orientation (rows <= cols): one tile of 16 rows x 128 columns per workgroup, straight through
+// registers; in X, 16 rows of a column block lie back to back (1 KB runs).
 __global__ void __launch_bounds__(256)
 normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, long strideX, int rows, int cols,
                  int Mp, int Kp) {
-    constexpr int TR = 64, TC = 128, PITCH = TC + 8;
+    constexpr int TR = 16, TC = 128;
+    const int b = blockIdx.y;
+    const float d = denom[b];
+    const bf16_t* u = U + b * strideU;
+    bf16_t* x = X + b * strideX;
+    const int cbx = Kp / BLK_COLS;
+    const int tiles_c = Kp / TC;
+    const int r = (blockIdx.x / tiles_c) * TR + (threadIdx.x >> 4), c = (blockIdx.x % tiles_c) * TC + (threadIdx.x & 15) * 8;
+    bf16x8 v;
+    if (r < rows && (cols % 8) == 0 && c + 8 <= cols) {
+        v = *(const bf16x8*)(u + (long)r * cols + c);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (r < rows && c + i < cols) ? u[(long)r * cols + c + i] : (bf16_t)0.f;
+    }
+    bf16x8 o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = f2bf(__fdiv_rn(bf2f(v[i]), d));
+    *(bf16x8*)(x + blocked_offset(r, c, cbx)) = o;
+}
+
+// A parameter with rows > cols (X = u^T): a tile of TR rows x TC columns of u goes through an LDS transpose and leaves
+// as TC rows of X, TR elements each (TR = 32: the 64-byte rows of one column block, TC of them back to back).
+template <int TR, int TC>
+__global__ void __launch_bounds__(256)
+normalize_t_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, long strideX, int rows, int cols,
+                   int Mp, int Kp) {
+    constexpr int PITCH = TC + 8;
+    constexpr int LCH = TC / 8, LROWS = 256 / LCH, LPASS = TR / LROWS;  // load: chunks per tile row, rows and passes
+    constexpr int SCH = TR / 8, SROWS = 256 / SCH, SPASS = TC / SROWS;  // store: chunks per X row, X rows and passes
+    static_assert(LPASS >= 1 && SPASS >= 1 && TR % 8 == 0 && TC % 8 == 0, "a whole number of passes");
     __shared__ __align__(16) bf16_t tile[TR][PITCH];
     const int b = blockIdx.y;
     const float d = denom[b];
     const bf16_t* u = U + b * strideU;
     bf16_t* x = X + b * strideX;
-    const bool transposed = rows > cols;
-    const int Cp = transposed ? Mp : Kp;  // padded columns of u's image
     const int cbx = Kp / BLK_COLS;
-    const int tiles_c = Cp / TC;
+    const int tiles_c = Mp / TC;  // u's padded image is Kp rows x Mp columns
     const int r0 = (blockIdx.x / tiles_c) * TR, c0 = (blockIdx.x % tiles_c) * TC;
-    const int tr = threadIdx.x >> 4, tc = (threadIdx.x & 15) * 8;  // 16 rows x 16 chunks per pass
+    const int tr = threadIdx.x / LCH, tc = (threadIdx.x % LCH) * 8;
     const bool vec = (cols % 8) == 0;
-    bf16x8 v[4];
 #pragma unroll
-    for (int h = 0; h < 4; ++h) {
-        const int r = r0 + tr + h * 16, c = c0 + tc;
+    for (int h = 0; h < LPASS; ++h) {
+        const int r = r0 + tr + h * LROWS, c = c0 + tc;
+        bf16x8 v;
         if (r < rows && vec && c + 8 <= cols) {
-            v[h] = *(const bf16x8*)(u + (long)r * cols + c);
+            v = *(const bf16x8*)(u + (long)r * cols + c);
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[h][i] = (r < rows && c + i < cols) ? u[(long)r * cols + c + i] : (bf16_t)0.f;
+            for (int i = 0; i < 8; ++i) v[i] = (r < rows && c + i < cols) ? u[(long)r * cols + c + i] : (bf16_t)0.f;
         }
-    }
-#pragma unroll
-    for (int h = 0; h < 4; ++h) {
-        const int r = r0 + tr + h * 16, c = c0 + tc;
         bf16x8 o;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] = f2bf(__fdiv_rn(bf2f(v[h][i]), d));
-        if (transposed) *(bf16x8*)(&tile[tr + h * 16][tc]) = o;
-        else *(bf16x8*)(x + blocked_offset(r, c, cbx)) = o;
+        for (int i = 0; i < 8; ++i) o[i] = f2bf(__fdiv_rn(bf2f(v[i]), d));
+        *(bf16x8*)(&tile[tr + h * LROWS][tc]) = o;
     }
-    if (!transposed) return;
     __syncthreads();
-    // X[c][r]: 128 rows of 64 elements; a thread gathers 8 consecutive r of one column of the tile
-    const int fr = (threadIdx.x & 7) * 8, fc0 = threadIdx.x >> 3;  // 8 chunks per row, 32 rows per pass
+    // X[c][r]: a thread gathers 8 consecutive r of one column of the tile
+    const int fr = (threadIdx.x % SCH) * 8, fc0 = threadIdx.x / SCH;
 #pragma unroll
-    for (int h = 0; h < 4; ++h) {
-        const int fc = fc0 + h * 32;
+    for (int h = 0; h < SPASS; ++h) {
+        const int fc = fc0 + h * SROWS;
         bf16x8 o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) o[i] = tile[fr + i][fc];
@@ -542,7 +580,7 @@ inline void lerp_consts(double weight, float& w, float& wm1, bool& small) {
 
 }  // namespace
 
-int momentum_parts(long n) { return blocks_for(n, 16384, MUON_MAX_PARTS); }
+int momentum_parts(long n) { return blocks_for(n, MUON_PART_ELEMS, MUON_MAX_PARTS); }
 
 hipError_t launch_momentum_norm(const void* const* g_ptrs, const void* const* m_ptrs, int g_dtype, int m_dtype,
                                 bf16_t* U, long strideU, float* partials, int nparts, long n, int batch,
@@ -585,9 +623,16 @@ hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials
                             long strideX, int rows, int cols, int Mp, int Kp, int batch, unsigned* clear, int clear_words,
                             hipStream_t stream) {
     hipLaunchKernelGGL(frob_finalize_kernel, dim3(batch), dim3(256), 0, stream, partials, nparts, denom, clear, clear_words);
-    // u's padded image is Rp x Cp with Rp a multiple of 64 and Cp a multiple of 128 (both are multiples of the tile edge)
-    dim3 grid((Mp / 64) * (Kp / 64) / 2, batch), block(256);
-    hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, strideX, rows, cols, Mp, Kp);
+    // u's padded image has whole 128-tiles in both directions (Mp and Kp are multiples of the GEMM tile edge)
+    if (rows > cols) {
+        // 32 x 128 measured best of {32, 64} x {64, 128}: 5.5 to 5.7 TB/s against 5.2 to 5.5 for 64 x 128
+        constexpr int TR = 32, TC = 128;
+        dim3 grid((Kp / TR) * (Mp / TC), batch), block(256);
+        hipLaunchKernelGGL((normalize_t_kernel<TR, TC>), grid, block, 0, stream, U, strideU, denom, X, strideX, rows, cols, Mp, Kp);
+    } else {
+        dim3 grid((Mp / 16) * (Kp / 128), batch), block(256);
+        hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, strideX, rows, cols, Mp, Kp);
+    }
     return hipGetLastError();
 }
 

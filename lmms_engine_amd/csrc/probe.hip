@@ -86,3 +86,38 @@ extern "C" __attribute__((visibility("default"))) int muon_probe_mfma(const void
     if (flop) *flop = MUON_PROBE_FLOP_PER_ITER * iters;
     return (int)hipGetLastError();
 }
+
+// Streaming rate of plain kernels against the number of XCDs that take part (workgroup b sits on XCD b % 8; the others
+// leave at once): what the memory system delivers for one read (mode 0), one read and one write in place (mode 1) and a
+// copy (mode 2), the ceilings the elementwise kernels of the step are read against.
+namespace {
+template <int MODE>
+__global__ void __launch_bounds__(256) stream_probe_kernel(f32x4* a, f32x4* b, long n4, int nx, float* sink) {
+    const int xcd = blockIdx.x & 7;
+    if (xcd >= nx) return;
+    const long wg = (long)(blockIdx.x >> 3) * nx + xcd, nwg = (long)(gridDim.x >> 3) * nx;
+    const long per = (n4 + nwg - 1) / nwg;
+    const long lo = wg * per, hi = lo + per < n4 ? lo + per : n4;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (long i = lo + threadIdx.x; i < hi; i += 256) {
+        const f32x4 v = a[i];
+        if (MODE == 0) acc += v;
+        else if (MODE == 1) a[i] = v * 1.0001f;
+        else b[i] = v;
+    }
+    if (MODE == 0 && acc[0] + acc[1] + acc[2] + acc[3] == 12345.f) *sink = 1.f;  // keeps the loads alive
+}
+}  // namespace
+
+// a, b: `bytes` of device memory each (a multiple of 16); mode 0, 1, 2 as above; xcds 1..8.  Returns a hipError_t or -1.
+extern "C" __attribute__((visibility("default"))) int muon_probe_stream(void* a, void* b, long bytes, int mode, int xcds, void* sink,
+                                                                        void* stream) {
+    if (!a || !b || !sink || bytes <= 0 || bytes % 16 || mode < 0 || mode > 2 || xcds < 1 || xcds > 8) return -1;
+    const long n4 = bytes / 16;
+    dim3 grid(8 * 2048), block(256);
+    hipStream_t s = (hipStream_t)stream;
+    if (mode == 0) hipLaunchKernelGGL(stream_probe_kernel<0>, grid, block, 0, s, (f32x4*)a, (f32x4*)b, n4, xcds, (float*)sink);
+    else if (mode == 1) hipLaunchKernelGGL(stream_probe_kernel<1>, grid, block, 0, s, (f32x4*)a, (f32x4*)b, n4, xcds, (float*)sink);
+    else hipLaunchKernelGGL(stream_probe_kernel<2>, grid, block, 0, s, (f32x4*)a, (f32x4*)b, n4, xcds, (float*)sink);
+    return (int)hipGetLastError();
+}
