@@ -529,7 +529,7 @@ int check_norm_kind(int k) {
 int check_list(const void* ptrs, const long* numel, const long* chunk_start, int n, long chunks, int dtype) {
     if (!ptrs || !numel || !chunk_start) return fail(MUON_HIP_EINVAL, "null tensor-list array");
     if (n <= 0 || chunks <= 0) return fail(MUON_HIP_EINVAL, "a tensor list needs at least one tensor and one chunk");
-    if (chunks > 0x7fffffffL) return fail(MUON_HIP_ESHAPE, "%ld chunks exceed one launch", chunks);
+    if (chunks > 0x1fffffffL) return fail(MUON_HIP_ESHAPE, "%ld chunks exceed one launch", chunks);  // up to four workgroups each
     if (!dtype_ok(dtype)) return fail(MUON_HIP_EINVAL, "unknown dtype %d", dtype);
     return 0;
 }
