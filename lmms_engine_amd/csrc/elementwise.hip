@@ -227,8 +227,7 @@ __global__ void __launch_bounds__(256) frob_finalize_kernel(const float* partial
 // A parameter in X's orientation (rows <= cols): one tile of 16 rows x 128 columns per workgroup, straight through
 // registers; in X, 16 rows of a column block lie back to back (1 KB runs).
 __global__ void __launch_bounds__(256)
-normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, long strideX, int rows, int cols,
-                 int Mp, int Kp) {
+normalize_kernel(const bf16_t* U, long strideU, const float* denom, bf16_t* X, long strideX, int rows, int cols, int Kp) {
     constexpr int TR = 16, TC = 128;
     const int b = blockIdx.y;
     const float d = denom[b];
@@ -631,7 +630,7 @@ hipError_t launch_normalize(const bf16_t* U, long strideU, const float* partials
         hipLaunchKernelGGL((normalize_t_kernel<TR, TC>), grid, block, 0, stream, U, strideU, denom, X, strideX, rows, cols, Mp, Kp);
     } else {
         dim3 grid((Mp / 16) * (Kp / 128), batch), block(256);
-        hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, strideX, rows, cols, Mp, Kp);
+        hipLaunchKernelGGL(normalize_kernel, grid, block, 0, stream, U, strideU, denom, X, strideX, rows, cols, Kp);
     }
     return hipGetLastError();
 }
