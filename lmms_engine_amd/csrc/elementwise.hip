@@ -564,6 +564,10 @@ __global__ void __launch_bounds__(256) decay_update_kernel(PT* p, const UT* u, l
         Ld<PT>::store(p + i, fmaf(alpha, Ld<UT>::load(u + i), Ld<PT>::rnd(Ld<PT>::load(p + i) * decay)));
 }
 
+// Grids of the helper kernels: enough workgroups that each makes one or two trips of its loop (short-lived workgroups
+// stream faster than a few thousand that loop), up to this many.
+constexpr int kMaxBlocks = 1 << 20;
+
 inline int blocks_for(long n, int per_block, int cap) {
     long b = (n + per_block - 1) / per_block;
     if (b < 1) b = 1;
@@ -655,7 +659,7 @@ hipError_t launch_apply_update(const void* const* p_ptrs, int p_dtype, const bf1
             return hipErrorInvalidValue;
         return hipGetLastError();
     }
-    dim3 grid(blocks_for((long)rows * cols, 16384, 8192), batch);
+    dim3 grid(blocks_for((long)rows * cols, 4096, kMaxBlocks), batch);
     if (p_dtype == MUON_HIP_F32)
         hipLaunchKernelGGL((apply_update_kernel<float>), grid, block, 0, stream, p_ptrs, O, strideO, cbo, rows, cols, um);
     else if (p_dtype == MUON_HIP_BF16)
@@ -699,7 +703,7 @@ AdamMath adam_math(int step, double lr, double b1, double b2, double eps, double
 hipError_t launch_adamw(void* p, const void* g, void* e1, void* e2, int dtype, long n, int step, double lr,
                         double b1, double b2, double eps, double wd, hipStream_t stream) {
     const AdamMath am = adam_math(step, lr, b1, b2, eps, wd);
-    dim3 grid(blocks_for(n, 256 * 4, 8192)), block(256);
+    dim3 grid(blocks_for(n, 256 * 4, kMaxBlocks)), block(256);
     if (dtype == MUON_HIP_F32)
         hipLaunchKernelGGL((adamw_kernel<float>), grid, block, 0, stream, (float*)p, (const float*)g, (float*)e1,
                            (float*)e2, n, am);
@@ -714,7 +718,7 @@ hipError_t launch_adamw(void* p, const void* g, void* e1, void* e2, int dtype, l
 hipError_t launch_adam_update(const void* g, void* e1, void* e2, void* out, int dtype, long n, int step, double b1,
                               double b2, double eps, hipStream_t stream) {
     const AdamMath am = adam_math(step, 0.0, b1, b2, eps, 0.0);
-    dim3 grid(blocks_for(n, 256 * 8 * 2, 8192)), block(256);
+    dim3 grid(blocks_for(n, 256 * 8 * 2, kMaxBlocks)), block(256);
     if (dtype == MUON_HIP_F32)
         hipLaunchKernelGGL((adam_update_kernel<float>), grid, block, 0, stream, (const float*)g, (float*)e1, (float*)e2,
                            (float*)out, n, am);
@@ -727,7 +731,7 @@ hipError_t launch_adam_update(const void* g, void* e1, void* e2, void* out, int 
 }
 
 hipError_t launch_scale(void* x, int dtype, long n, double s, hipStream_t stream) {
-    dim3 grid(blocks_for(n, 256 * 8 * 2, 8192)), block(256);
+    dim3 grid(blocks_for(n, 256 * 8 * 2, kMaxBlocks)), block(256);
     if (dtype == MUON_HIP_F32) hipLaunchKernelGGL((scale_kernel<float>), grid, block, 0, stream, (float*)x, n, (float)s);
     else if (dtype == MUON_HIP_BF16) hipLaunchKernelGGL((scale_kernel<bf16_t>), grid, block, 0, stream, (bf16_t*)x, n, (float)s);
     else return hipErrorInvalidValue;
@@ -737,7 +741,7 @@ hipError_t launch_scale(void* x, int dtype, long n, double s, hipStream_t stream
 hipError_t launch_decay_update(void* p, int p_dtype, const void* u, int u_dtype, long n, double lr, double wd,
                                hipStream_t stream) {
     const float decay = (float)(1.0 - lr * wd), alpha = (float)(-lr);
-    dim3 grid(blocks_for(n, 256 * 8 * 2, 8192)), block(256);
+    dim3 grid(blocks_for(n, 256 * 8 * 2, kMaxBlocks)), block(256);
     if (p_dtype == MUON_HIP_F32 && u_dtype == MUON_HIP_F32)
         hipLaunchKernelGGL((decay_update_kernel<float, float>), grid, block, 0, stream, (float*)p, (const float*)u, n, decay, alpha);
     else if (p_dtype == MUON_HIP_F32 && u_dtype == MUON_HIP_BF16)
