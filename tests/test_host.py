@@ -326,3 +326,47 @@ def test_chunk_choice_lands_on_whole_rounds():
     for n, cap, rows, cols in ((72, 15, 4096, 4096), (72, 7, 12288, 4096), (36, 7, 4096, 12288), (24, 91, 896, 4864)):
         nb = pick(n, cap, rows, cols)
         assert 1 <= nb <= min(n, cap)
+
+
+def test_persistent_tile_handout_model():
+    """A host model of how the persistent GEMM kernel hands out tiles (csrc/gemm_nt.hip: two static rounds per workgroup,
+    then one atomic counter per XCD; virtual ids mapped to tiles by xcd_remap of csrc/common.h), for device shapes other
+    than the 256 compute units / 8 XCDs of a whole MI355X as well: whatever order the workgroups ask in, every tile is
+    computed exactly once, and a counter never hands out more than one id past the end per workgroup."""
+    import random
+
+    XCD_CHUNK = 32
+
+    def xcd_remap(pid, nblocks, shift):
+        span = XCD_CHUNK << shift
+        full = nblocks // span * span
+        if pid >= full:
+            return pid
+        xcd, local = pid & ((1 << shift) - 1), pid >> shift
+        return (((local // XCD_CHUNK) << shift) + xcd) * XCD_CHUNK + local % XCD_CHUNK
+
+    rng = random.Random(7)
+    for cus, shift in ((256, 3), (128, 2), (64, 1), (32, 0), (304, 3)):
+        for total in (cus + 1, 2 * cus, 2 * cus + 1, 5 * cus + 37, 17 * cus, 9216):
+            grid = min(total, cus)
+            assert grid % (1 << shift) == 0
+            # the remap is a bijection of the virtual ids onto the tiles
+            assert sorted(xcd_remap(p, total, shift) for p in range(total)) == list(range(total))
+            counters = [0] * (1 << shift)
+            done = []
+            # workgroup state: (current id, next id); a workgroup asks for the id after next while it has a next tile
+            wgs = {b: [b, b + grid] for b in range(grid)}
+            active = list(wgs)
+            while active:
+                b = rng.choice(active)  # any interleaving
+                cur, nxt = wgs[b]
+                done.append(cur)
+                if nxt >= total:
+                    active.remove(b)
+                    continue
+                xcd = b & ((1 << shift) - 1)
+                fetched = counters[xcd]
+                counters[xcd] += 1
+                wgs[b] = [nxt, ((2 * (grid >> shift) + fetched) << shift) + xcd]
+            assert sorted(done) == list(range(total)), (cus, shift, total)
+            assert sum(counters) <= total  # bounded: nobody spins on the counters
