@@ -212,9 +212,10 @@ int muon_hip_adamw_multi(const void* const* p_ptrs, const void* const* g_ptrs, c
                          double beta1, double beta2, double eps, double weight_decay, void* stream);
 
 /* Gradient clipping, the step before optimizer.step(): fsdp2_clip_grad_norm_ on one device
- * (utils/fsdp2_utils.py:234-255) is torch's _get_total_norm + _clip_grads_with_norm_.  `norm_kind` is
- * MUON_HIP_NORM_L2 (norm_type 2, the default of the reference) or MUON_HIP_NORM_INF (norm_type inf: the largest
- * magnitude; a NaN anywhere makes the result NaN, as torch's max does).
+ * (utils/fsdp2_utils.py:234-255) is torch's _get_total_norm + _clip_grads_with_norm_.  `norm_type` is the
+ * reference's argument of that name, with the meanings torch.linalg.vector_norm gives it: 2 (the default), 1,
+ * 0 (the count of non-zeros), +inf / -inf (the largest / smallest magnitude; a NaN anywhere makes the result NaN,
+ * as torch's max and min do) and any other order p as (sum |x|^p)^(1/p) in fp32.  NaN is rejected.
  * muon_hip_grad_norms: norms[t] = ||g_t|| accumulated in fp32 and rounded to the tensors' dtype,
  *   as fp32 values (the per-tensor norms of torch._foreach_norm); `partials` is scratch of
  *   `chunks` floats.
@@ -223,11 +224,9 @@ int muon_hip_adamw_multi(const void* const* p_ptrs, const void* const* g_ptrs, c
  * muon_hip_clip_scale: g_t *= min(1, max_norm / (total + 1e-6)) for every tensor of the list,
  *   the coefficient evaluated as torch does, (total + 1e-6).reciprocal() * max_norm in the
  *   norm's dtype `norm_dtype`, read from device memory so that no host synchronisation is needed. */
-#define MUON_HIP_NORM_L2 0
-#define MUON_HIP_NORM_INF 1
 int muon_hip_grad_norms(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
-                        int dtype, int norm_kind, float* partials, float* norms, void* stream);
-int muon_hip_total_norm(const float* norms, int n, int dtype, int norm_kind, float* total_f32, void* total_typed,
+                        int dtype, double norm_type, float* partials, float* norms, void* stream);
+int muon_hip_total_norm(const float* norms, int n, int dtype, double norm_type, float* total_f32, void* total_typed,
                         void* stream);
 
 /* muon_hip_grad_norms without the `partials` argument.  No counterpart in the reference: it is for callers
@@ -239,7 +238,7 @@ int muon_hip_total_norm(const float* norms, int n, int dtype, int norm_kind, flo
  * them.  The first call on a device looks the array's address up and must not run under stream capture. */
 #define MUON_HIP_STATIC_MAX_CHUNKS (1 << 20)
 int muon_hip_grad_norms_static(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n,
-                               long chunks, int dtype, int norm_kind, float* norms, void* stream);
+                               long chunks, int dtype, double norm_type, float* norms, void* stream);
 int muon_hip_clip_scale(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
                         int dtype, const float* total_f32, int norm_dtype, double max_norm, void* stream);
 

@@ -23,7 +23,6 @@ KERNEL_NAMES = ["momentum_norm", "normalize", "syrk", "sympoly", "bx_axpy", "app
 MULTI_CHUNK = 16384  # MUON_HIP_MULTI_CHUNK
 STATIC_MAX_CHUNKS = 1 << 20  # MUON_HIP_STATIC_MAX_CHUNKS
 PPX_COUNTER_BYTES = 576  # MUON_HIP_PPX_COUNTER_BYTES
-NORM_L2, NORM_INF = 0, 1  # MUON_HIP_NORM_*
 
 # name -> (restype, argtypes); mirrors include/muon_hip.h one to one
 SIGNATURES = {
@@ -57,9 +56,9 @@ SIGNATURES = {
     "muon_hip_scale": (c_int, [c_void_p, c_int, c_long, c_double, c_void_p]),
     "muon_hip_decay_update": (c_int, [c_void_p, c_int, c_void_p, c_int, c_long, c_double, c_double, c_void_p]),
     "muon_hip_adamw_multi": (c_int, [c_void_p] * 8 + [c_int, c_long, c_int] + [c_double] * 5 + [c_void_p]),
-    "muon_hip_grad_norms": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p]),
-    "muon_hip_grad_norms_static": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_int, c_void_p, c_void_p]),
-    "muon_hip_total_norm": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "muon_hip_grad_norms": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_void_p, c_void_p, c_void_p]),
+    "muon_hip_grad_norms_static": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_double, c_void_p, c_void_p]),
+    "muon_hip_total_norm": (c_int, [c_void_p, c_int, c_int, c_double, c_void_p, c_void_p, c_void_p]),
     "muon_hip_clip_scale": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_long, c_int, c_void_p, c_int, c_double,
                                     c_void_p]),
     "muon_hip_device_shape": (c_int, [POINTER(c_int), POINTER(c_int)]),

@@ -19,20 +19,16 @@ from .multi_tensor import TensorListTable
 @torch.no_grad()
 def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=False, foreach=None) -> Tensor:
     """Same signature and return value (the total norm, a 0-d tensor on the gradients' device) as
-    fsdp2_clip_grad_norm_.  norm_type 2 (the default) and inf have kernels, both bit-identical to torch's result in
-    bf16; other orders would need a power function whose roundings differ from torch's and are refused.  `foreach` is
-    accepted and ignored (every call is one launch per dtype)."""
+    fsdp2_clip_grad_norm_.  `norm_type` is any order torch.linalg.vector_norm takes: 2 (the default), 1, 0, inf and
+    -inf have reductions of their own, every other p is (sum |x|^p)^(1/p) accumulated in fp32 as torch does.
+    `foreach` is accepted and ignored (every call is one launch per dtype)."""
     if isinstance(parameters, Tensor):
         parameters = [parameters]
     else:
         parameters = list(parameters)
     norm_type = float(norm_type)
-    if norm_type == 2.0:
-        kind = _abi.NORM_L2
-    elif norm_type == float("inf"):
-        kind = _abi.NORM_INF
-    else:
-        raise NotImplementedError(f"norm_type 2 and inf have HIP kernels (got {norm_type})")
+    if norm_type != norm_type:
+        raise ValueError("norm_type is NaN")
     grads = [p.grad for p in parameters if p.grad is not None]
     if len(grads) == 0:
         return torch.tensor(0.0)  # what _get_total_norm returns for an empty list
@@ -65,12 +61,12 @@ def clip_grad_norm_(parameters, max_norm, norm_type=2.0, error_if_nonfinite=Fals
             if tab.chunks > 0:
                 partials = torch.empty(tab.chunks, dtype=torch.float32, device=dev)
                 _abi.check(lib.muon_hip_grad_norms(tab.role_ptrs[0], tab.numel_ptr, tab.chunk_start_ptr, tab.n, tab.chunks,
-                                                   _abi.dtype_code(dt), kind, partials.data_ptr(), norms.data_ptr() + 4 * off, s),
+                                                   _abi.dtype_code(dt), norm_type, partials.data_ptr(), norms.data_ptr() + 4 * off, s),
                            "grad_norms")
             else:
                 norms[off:off + tab.n].zero_()
             off += tab.n
-        _abi.check(lib.muon_hip_total_norm(norms.data_ptr(), n_total, _abi.dtype_code(out_dtype), kind, total_f32.data_ptr(),
+        _abi.check(lib.muon_hip_total_norm(norms.data_ptr(), n_total, _abi.dtype_code(out_dtype), norm_type, total_f32.data_ptr(),
                                            total.data_ptr(), s), "total_norm")
         if error_if_nonfinite and not bool(torch.isfinite(total)):
             raise RuntimeError(

@@ -522,8 +522,8 @@ int muon_hip_decay_update(void* p, int p_dtype, const void* u, int u_dtype, long
 }
 
 namespace {
-int check_norm_kind(int k) {
-    if (k != MUON_HIP_NORM_L2 && k != MUON_HIP_NORM_INF) return fail(MUON_HIP_EINVAL, "norm kind %d is neither the 2-norm nor the infinity norm", k);
+int check_norm_type(double norm_type) {
+    if (norm_type != norm_type) return fail(MUON_HIP_EINVAL, "norm_type is NaN");
     return 0;
 }
 int check_list(const void* ptrs, const long* numel, const long* chunk_start, int n, long chunks, int dtype) {
@@ -550,14 +550,14 @@ int muon_hip_adamw_multi(const void* const* p_ptrs, const void* const* g_ptrs, c
 }
 
 int muon_hip_grad_norms(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, long chunks,
-                        int dtype, int norm_kind, float* partials, float* norms, void* stream) {
+                        int dtype, double norm_type, float* partials, float* norms, void* stream) {
     if (int rc = check_list(g_ptrs, numel, chunk_start, n, chunks, dtype)) return rc;
-    if (int rc = check_norm_kind(norm_kind)) return rc;
+    if (int rc = check_norm_type(norm_type)) return rc;
     if (!partials || !norms) return fail(MUON_HIP_EINVAL, "null output");
     hipStream_t s = (hipStream_t)stream;
     Timed t(MUON_HIP_K_GRAD_NORM, s);
     const MultiTensorList l{g_ptrs, numel, chunk_start, n, chunks};
-    hipError_t e = launch_tensor_norms(l, dtype, norm_kind == MUON_HIP_NORM_INF, partials, norms, s);
+    hipError_t e = launch_tensor_norms(l, dtype, norm_type, partials, norms, s);
     return e == hipSuccess ? 0 : hip_fail(e, "grad_norms launch");
 }
 
@@ -591,9 +591,9 @@ int scratch_for_current_device(float** out) {
 }  // namespace
 
 int muon_hip_grad_norms_static(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n,
-                               long chunks, int dtype, int norm_kind, float* norms, void* stream) {
+                               long chunks, int dtype, double norm_type, float* norms, void* stream) {
     if (int rc = check_list(g_ptrs, numel, chunk_start, n, chunks, dtype)) return rc;
-    if (int rc = check_norm_kind(norm_kind)) return rc;
+    if (int rc = check_norm_type(norm_type)) return rc;
     if (!norms) return fail(MUON_HIP_EINVAL, "null output");
     if (chunks > (long)MUON_HIP_STATIC_MAX_CHUNKS)
         return fail(MUON_HIP_ESHAPE, "%ld chunks exceed the %ld the built-in scratch array holds; use muon_hip_grad_norms "
@@ -604,16 +604,16 @@ int muon_hip_grad_norms_static(const void* const* g_ptrs, const long* numel, con
     Timed t(MUON_HIP_K_GRAD_NORM, s);
     const MultiTensorList l{g_ptrs, numel, chunk_start, n, chunks};
     // every partial the second kernel reads is written by the first: nothing has to start at zero
-    hipError_t e = launch_tensor_norms(l, dtype, norm_kind == MUON_HIP_NORM_INF, partials, norms, s);
+    hipError_t e = launch_tensor_norms(l, dtype, norm_type, partials, norms, s);
     return e == hipSuccess ? 0 : hip_fail(e, "grad_norms launch");
 }
 
-int muon_hip_total_norm(const float* norms, int n, int dtype, int norm_kind, float* total_f32, void* total_typed,
+int muon_hip_total_norm(const float* norms, int n, int dtype, double norm_type, float* total_f32, void* total_typed,
                         void* stream) {
     if (!norms || !total_f32 || !total_typed || n <= 0 || !dtype_ok(dtype))
         return fail(MUON_HIP_EINVAL, "null pointer, empty list or unknown dtype");
-    if (int rc = check_norm_kind(norm_kind)) return rc;
-    hipError_t e = launch_total_norm(norms, n, dtype, norm_kind == MUON_HIP_NORM_INF, total_f32, total_typed,
+    if (int rc = check_norm_type(norm_type)) return rc;
+    hipError_t e = launch_total_norm(norms, n, dtype, norm_type, total_f32, total_typed,
                                      (hipStream_t)stream);
     return e == hipSuccess ? 0 : hip_fail(e, "total_norm launch");
 }

@@ -4,8 +4,9 @@
 //                      :468-477) for every tensor of a parameter group
 //   sqnorm / norms   : the norm torch's _get_total_norm computes for
 //                      fsdp2_clip_grad_norm_ (utils/fsdp2_utils.py:234-255): per-tensor norms
-//                      rounded to the tensor dtype, then the norm of those norms; the 2-norm, or the
-//                      infinity norm (largest magnitude, a NaN anywhere makes the result NaN, as torch's max does)
+//                      rounded to the tensor dtype, then the norm of those norms, for any order torch's
+//                      vector_norm takes: 2, 1, 0 (count of non-zeros), +inf / -inf (largest / smallest magnitude,
+//                      a NaN anywhere makes the result NaN, as torch's max and min do), and (sum |x|^p)^(1/p) otherwise
 //   clip_scale_multi : _clip_grads_with_norm_: g *= clamp(max_norm / (total + 1e-6), max=1)
 //
 // A tensor list is cut into chunks of MUON_MULTI_CHUNK elements; chunk_start[t] is the index of
@@ -13,6 +14,7 @@
 // tensor by bisection and handles one chunk: 16-byte vectors when every base pointer of the
 // tensor is 16-byte aligned, scalars otherwise and for the last few elements.
 #include "multi_tensor.h"
+#include <type_traits>
 
 namespace {
 
@@ -155,66 +157,96 @@ __device__ __forceinline__ float block_sum_256(float v, float* red) {
     return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
-// Largest of two magnitudes; a NaN on either side wins (fmaxf would drop it).
+// Largest / smallest of two magnitudes; a NaN on either side wins (fmaxf and fminf would drop it).
 __device__ __forceinline__ float nan_max(float a, float b) { return (a != a) ? a : (b != b) ? b : fmaxf(a, b); }
+__device__ __forceinline__ float nan_min(float a, float b) { return (a != a) ? a : (b != b) ? b : fminf(a, b); }
 
-__device__ __forceinline__ float block_max_256(float v, float* red) {
+// The reductions of torch's norm kernels (aten/src/ATen/native/cuda/ReduceNormKernel.cu and SharedReduceOps.h), by order:
+// what one element adds to the running value, how two running values combine, and what turns the total into the norm.
+enum NormKind { NORM_TWO, NORM_INF, NORM_ONE, NORM_ZERO, NORM_NEG_INF, NORM_P };
+
+template <int KIND> struct NormOp {
+    static constexpr bool kSum = KIND != NORM_INF && KIND != NORM_NEG_INF;
+    static __device__ __forceinline__ float identity() { return KIND == NORM_NEG_INF ? __builtin_inff() : 0.f; }
+    static __device__ __forceinline__ float reduce(float acc, float v, float p) {
+        if constexpr (KIND == NORM_TWO) return fmaf(v, v, acc);
+        else if constexpr (KIND == NORM_INF) return nan_max(acc, fabsf(v));
+        else if constexpr (KIND == NORM_NEG_INF) return nan_min(acc, fabsf(v));
+        else if constexpr (KIND == NORM_ONE) return acc + fabsf(v);
+        else if constexpr (KIND == NORM_ZERO) return acc + (v == 0.f ? 0.f : 1.f);
+        else return acc + powf(fabsf(v), p);
+    }
+    static __device__ __forceinline__ float combine(float a, float b) {
+        if constexpr (KIND == NORM_INF) return nan_max(a, b);
+        else if constexpr (KIND == NORM_NEG_INF) return nan_min(a, b);
+        else return a + b;
+    }
+    static __device__ __forceinline__ float project(float acc, float p) {
+        if constexpr (KIND == NORM_TWO) return sqrtf(acc);
+        else if constexpr (KIND == NORM_P) return powf(acc, __fdiv_rn(1.0f, p));
+        else return acc;
+    }
+};
+
+template <int KIND>
+__device__ __forceinline__ float block_reduce_256(float v, float* red) {
+    if constexpr (NormOp<KIND>::kSum) {
+        return block_sum_256(v, red);
+    } else {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v = nan_max(v, __shfl_xor(v, off, 64));
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    __syncthreads();
-    if (lane == 0) red[wave] = v;
-    __syncthreads();
-    return nan_max(nan_max(red[0], red[1]), nan_max(red[2], red[3]));
+        for (int off = 32; off > 0; off >>= 1) v = NormOp<KIND>::combine(v, __shfl_xor(v, off, 64));
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        __syncthreads();
+        if (lane == 0) red[wave] = v;
+        __syncthreads();
+        return NormOp<KIND>::combine(NormOp<KIND>::combine(red[0], red[1]), NormOp<KIND>::combine(red[2], red[3]));
+    }
 }
 
-// INF = false: sum of squares of a chunk; true: its largest magnitude.
-template <typename T, bool INF>
+// The running value of one chunk (sum of squares, of magnitudes, of powers, the count of non-zeros, or the extreme magnitude).
+template <typename T, int KIND>
 __global__ void __launch_bounds__(256)
-sqnorm_multi_kernel(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, float* partials) {
+sqnorm_multi_kernel(const void* const* g_ptrs, const long* numel, const long* chunk_start, int n, float p, float* partials) {
     __shared__ float red[4];
     const ChunkRange r = my_chunk(numel, chunk_start, n);
     const T* g = (const T*)g_ptrs[r.t] + r.begin;
     const bool vec = (((uintptr_t)g) & 15) == 0;
     const long n8 = vec ? r.len / 8 : 0;
-    float ss = 0.f;
+    float ss = NormOp<KIND>::identity();
     for (long i = threadIdx.x; i < n8; i += 256) {
         float v[8];
         Mt<T>::load8(g + i * 8, v);
 #pragma unroll
-        for (int k = 0; k < 8; ++k) ss = INF ? nan_max(ss, fabsf(v[k])) : fmaf(v[k], v[k], ss);
+        for (int k = 0; k < 8; ++k) ss = NormOp<KIND>::reduce(ss, v[k], p);
     }
-    for (long i = n8 * 8 + threadIdx.x; i < r.len; i += 256) {
-        const float v = Mt<T>::load(g + i);
-        ss = INF ? nan_max(ss, fabsf(v)) : fmaf(v, v, ss);
-    }
-    ss = INF ? block_max_256(ss, red) : block_sum_256(ss, red);
+    for (long i = n8 * 8 + threadIdx.x; i < r.len; i += 256) ss = NormOp<KIND>::reduce(ss, Mt<T>::load(g + i), p);
+    ss = block_reduce_256<KIND>(ss, red);
     if (threadIdx.x == 0) partials[blockIdx.x] = ss;
 }
 
 // One block per tensor: its partial results in a fixed order -> norm, rounded to the tensor dtype.
-template <bool INF>
+template <int KIND>
 __global__ void __launch_bounds__(256)
-tensor_norm_kernel(const float* partials, const long* chunk_start, int dtype, float* norms) {
+tensor_norm_kernel(const float* partials, const long* chunk_start, int dtype, float p, float* norms) {
     __shared__ float red[4];
     const int t = blockIdx.x;
-    float ss = 0.f;
-    for (long c = chunk_start[t] + threadIdx.x; c < chunk_start[t + 1]; c += 256) ss = INF ? nan_max(ss, partials[c]) : ss + partials[c];
-    ss = INF ? block_max_256(ss, red) : block_sum_256(ss, red);
-    if (threadIdx.x == 0) norms[t] = INF ? ss : rnd_dtype(sqrtf(ss), dtype);
+    float ss = NormOp<KIND>::identity();
+    for (long c = chunk_start[t] + threadIdx.x; c < chunk_start[t + 1]; c += 256) ss = NormOp<KIND>::combine(ss, partials[c]);
+    ss = block_reduce_256<KIND>(ss, red);
+    if (threadIdx.x == 0) norms[t] = rnd_dtype(NormOp<KIND>::project(ss, p), dtype);
 }
 
 // One block: norm of the per-tensor norms, rounded to the result dtype; written as fp32 (for the
 // scaling kernel) and in the result dtype (the tensor the caller returns).
-template <bool INF>
+template <int KIND>
 __global__ void __launch_bounds__(256)
-total_norm_kernel(const float* norms, int n, int dtype, float* total_f32, void* total_typed) {
+total_norm_kernel(const float* norms, int n, int dtype, float p, float* total_f32, void* total_typed) {
     __shared__ float red[4];
-    float ss = 0.f;
-    for (int t = threadIdx.x; t < n; t += 256) ss = INF ? nan_max(ss, norms[t]) : fmaf(norms[t], norms[t], ss);
-    ss = INF ? block_max_256(ss, red) : block_sum_256(ss, red);
+    float ss = NormOp<KIND>::identity();
+    for (int t = threadIdx.x; t < n; t += 256) ss = NormOp<KIND>::reduce(ss, norms[t], p);
+    ss = block_reduce_256<KIND>(ss, red);
     if (threadIdx.x == 0) {
-        const float tn = INF ? ss : rnd_dtype(sqrtf(ss), dtype);
+        const float tn = rnd_dtype(NormOp<KIND>::project(ss, p), dtype);
         *total_f32 = tn;
         if (dtype == MUON_HIP_BF16) *(bf16_t*)total_typed = f2bf(tn);
         else *(float*)total_typed = tn;
@@ -278,25 +310,58 @@ hipError_t launch_adamw_multi(const MultiTensorList& l, const void* const* g_ptr
     return hipGetLastError();
 }
 
-hipError_t launch_tensor_norms(const MultiTensorList& l, int dtype, bool inf_norm, float* partials, float* norms,
+namespace {
+int norm_kind_of(double norm_type) {
+    if (norm_type == 2.0) return NORM_TWO;
+    if (norm_type == 1.0) return NORM_ONE;
+    if (norm_type == 0.0) return NORM_ZERO;
+    if (norm_type == (double)__builtin_inff()) return NORM_INF;
+    if (norm_type == -(double)__builtin_inff()) return NORM_NEG_INF;
+    return NORM_P;
+}
+
+// f(std::integral_constant<int, KIND>) for the kind of `norm_type`
+template <typename F> void with_norm_kind(double norm_type, F&& f) {
+    switch (norm_kind_of(norm_type)) {
+        case NORM_TWO: f(std::integral_constant<int, NORM_TWO>()); break;
+        case NORM_INF: f(std::integral_constant<int, NORM_INF>()); break;
+        case NORM_ONE: f(std::integral_constant<int, NORM_ONE>()); break;
+        case NORM_ZERO: f(std::integral_constant<int, NORM_ZERO>()); break;
+        case NORM_NEG_INF: f(std::integral_constant<int, NORM_NEG_INF>()); break;
+        default: f(std::integral_constant<int, NORM_P>()); break;
+    }
+}
+}  // namespace
+
+hipError_t launch_tensor_norms(const MultiTensorList& l, int dtype, double norm_type, float* partials, float* norms,
                                hipStream_t stream) {
     dim3 grid((unsigned)l.chunks), block(256);
     if (dtype != MUON_HIP_F32 && dtype != MUON_HIP_BF16) return hipErrorInvalidValue;
-    const bool f32 = dtype == MUON_HIP_F32;
-    auto k = f32 ? (inf_norm ? sqnorm_multi_kernel<float, true> : sqnorm_multi_kernel<float, false>)
-                 : (inf_norm ? sqnorm_multi_kernel<bf16_t, true> : sqnorm_multi_kernel<bf16_t, false>);
-    hipLaunchKernelGGL(k, grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n, partials);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    auto k2 = inf_norm ? tensor_norm_kernel<true> : tensor_norm_kernel<false>;
-    hipLaunchKernelGGL(k2, dim3((unsigned)l.n), block, 0, stream, partials, l.chunk_start, dtype, norms);
-    return hipGetLastError();
+    if (norm_type != norm_type) return hipErrorInvalidValue;
+    const float p = (float)norm_type;  // torch narrows the order to the accumulation type
+    hipError_t e = hipSuccess;
+    with_norm_kind(norm_type, [&](auto kind) {
+        constexpr int KIND = decltype(kind)::value;
+        if (dtype == MUON_HIP_F32)
+            hipLaunchKernelGGL((sqnorm_multi_kernel<float, KIND>), grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n, p, partials);
+        else
+            hipLaunchKernelGGL((sqnorm_multi_kernel<bf16_t, KIND>), grid, block, 0, stream, l.ptrs, l.numel, l.chunk_start, l.n, p, partials);
+        e = hipGetLastError();
+        if (e != hipSuccess) return;
+        hipLaunchKernelGGL((tensor_norm_kernel<KIND>), dim3((unsigned)l.n), block, 0, stream, partials, l.chunk_start, dtype, p, norms);
+        e = hipGetLastError();
+    });
+    return e;
 }
 
-hipError_t launch_total_norm(const float* norms, int n, int dtype, bool inf_norm, float* total_f32, void* total_typed,
+hipError_t launch_total_norm(const float* norms, int n, int dtype, double norm_type, float* total_f32, void* total_typed,
                              hipStream_t stream) {
-    auto k = inf_norm ? total_norm_kernel<true> : total_norm_kernel<false>;
-    hipLaunchKernelGGL(k, dim3(1), dim3(256), 0, stream, norms, n, dtype, total_f32, total_typed);
+    if (norm_type != norm_type) return hipErrorInvalidValue;
+    const float p = (float)norm_type;
+    with_norm_kind(norm_type, [&](auto kind) {
+        constexpr int KIND = decltype(kind)::value;
+        hipLaunchKernelGGL((total_norm_kernel<KIND>), dim3(1), dim3(256), 0, stream, norms, n, dtype, p, total_f32, total_typed);
+    });
     return hipGetLastError();
 }
 

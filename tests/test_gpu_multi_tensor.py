@@ -134,8 +134,8 @@ def test_clip_grad_norm_edge_cases(env):
         clip.clip_grad_norm_([p], 1.0, error_if_nonfinite=True)
     out = clip.clip_grad_norm_([p], 1.0)  # scales by the non-finite norm, as torch does
     assert torch.isinf(out) and torch.isnan(p.grad).all()
-    with pytest.raises(NotImplementedError):
-        clip.clip_grad_norm_([p], 1.0, norm_type=1.0)
+    with pytest.raises(ValueError):
+        clip.clip_grad_norm_([p], 1.0, norm_type=float("nan"))
     p.grad = torch.tensor([1.0, float("nan"), 3.0] + [0.0] * 7, device=dev)
     assert torch.isnan(clip.clip_grad_norm_([p], 1.0, norm_type=float("inf")))  # a NaN is the largest, as in torch.max
     q = torch.nn.Parameter(torch.zeros(4))
@@ -188,6 +188,45 @@ def test_clip_grad_norm_infinity_norm_and_strided_gradients(env, dtypes):
                 assert rel_fro(p.grad, c.grad) <= 1e-6
             else:
                 assert torch.equal(p.grad.cpu(), c.grad)
+
+
+@pytest.mark.parametrize("dtypes", [(torch.float32,), (torch.bfloat16,), (torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("norm_type", [1.0, 0.0, float("-inf"), 3.0, 0.5, 1.5])
+def test_clip_grad_norm_other_orders(env, dtypes, norm_type):
+    """Every other order fsdp2_clip_grad_norm_ can forward (utils/fsdp2_utils.py:244-254): the reductions of
+    torch.linalg.vector_norm by order (sum of magnitudes, count of non-zeros, smallest magnitude, (sum |x|^p)^(1/p)),
+    per tensor in fp32 rounded to the tensor's dtype, then over the per-tensor norms.  Against torch on the CPU: the
+    count and the smallest magnitude exactly; the sums to 1e-5 in fp32 (another order of additions, another power
+    routine) and to one bf16 step where the result is rounded to bf16."""
+    print("clip order", norm_type, dtypes, flush=True)
+    clip, dev = env["clip"], env["dev"]
+    gen = torch.Generator().manual_seed(43)
+    shapes = [(300, 70), (16384 * 2 + 5,), (9,), (64, 33), (3, 16384)]
+    ps, cpu = [], []
+    for i, s in enumerate(shapes):
+        dt = dtypes[i % len(dtypes)]
+        g = (0.5 * torch.randn(*s, generator=gen)).to(dt)
+        g.view(-1)[::7] = 0  # zeros for the count; the smallest magnitude is then 0 for the larger tensors
+        if i == 2:
+            g = g.abs() + 0.25  # one tensor without zeros
+        p, c = torch.nn.Parameter(torch.zeros(*s, dtype=dt, device=dev)), torch.nn.Parameter(torch.zeros(*s, dtype=dt))
+        p.grad, c.grad = g.to(dev), g.clone()
+        ps.append(p)
+        cpu.append(c)
+    for max_norm in (0.75, 1e9):
+        got = clip.clip_grad_norm_(ps, max_norm, norm_type=norm_type)
+        ref = torch.nn.utils.clip_grad_norm_(cpu, max_norm, norm_type=norm_type, foreach=False)
+        torch.cuda.synchronize()
+        assert got.dtype == ref.dtype
+        if norm_type in (0.0, float("-inf")):
+            assert got.item() == ref.item(), (norm_type, got.item(), ref.item())
+        else:
+            tol = 2.0 ** -7 if got.dtype == torch.bfloat16 else 1e-5
+            assert abs(got.item() - ref.item()) <= tol * abs(ref.item()), (norm_type, got.item(), ref.item())
+        for p, c in zip(ps, cpu):
+            tol = 2.0 ** -6 if torch.bfloat16 in dtypes else 2e-5   # the coefficient is rounded to the norm's dtype
+            assert rel_fro(p.grad, c.grad) <= tol, (norm_type, rel_fro(p.grad, c.grad))
+            c.grad.copy_(p.grad.cpu())  # both sides go on from the same gradients
 
 
 def test_clip_grad_norm_full_size(env):

@@ -221,7 +221,7 @@ def test_host_only_entry_points():
 
 def test_clip_grad_norm_host_behaviour():
     """What clip_grad_norm_ decides before any kernel runs: the empty cases return what torch's
-    _get_total_norm returns, other norms and CPU gradients are refused (no fallback path)."""
+    _get_total_norm returns, a NaN order and CPU gradients are refused (no fallback path)."""
     from lmms_engine_amd import _abi, clip_grad
 
     out = clip_grad.clip_grad_norm_([], 1.0)
@@ -229,10 +229,11 @@ def test_clip_grad_norm_host_behaviour():
     p = torch.nn.Parameter(torch.zeros(4))
     assert clip_grad.clip_grad_norm_(p, 1.0).item() == 0.0  # a bare tensor is accepted; no grad yet
     p.grad = torch.ones(4)
-    with pytest.raises(NotImplementedError):
-        clip_grad.clip_grad_norm_([p], 1.0, norm_type=3.0)
-    with pytest.raises(_abi.MuonHipError):
-        clip_grad.clip_grad_norm_([p], 1.0, norm_type=float("inf"))
+    with pytest.raises(ValueError):
+        clip_grad.clip_grad_norm_([p], 1.0, norm_type=float("nan"))
+    for norm_type in (3.0, 1.0, float("inf")):
+        with pytest.raises(_abi.MuonHipError):
+            clip_grad.clip_grad_norm_([p], 1.0, norm_type=norm_type)
     with pytest.raises(_abi.MuonHipError):
         clip_grad.clip_grad_norm_([p], 1.0)
     assert torch.equal(p.grad, torch.ones(4))  # untouched
@@ -300,18 +301,18 @@ def test_argument_errors_are_reported_before_any_launch():
                                       None), EINVAL, "at least one tensor")
     rejected(lib.muon_hip_adamw_multi(tbl, tbl, tbl, tbl, tbl, tbl, None, tbl, 1, 1, F32, 1e-3, 0.9, 0.95, 1e-8, 0.0,
                                       None), EINVAL, "null table")
-    rejected(lib.muon_hip_grad_norms(tbl, tbl, None, 1, 1, F32, 0, tbl, tbl, None), EINVAL, "null tensor-list")
-    rejected(lib.muon_hip_grad_norms(tbl, tbl, tbl, 1, 1, F32, 0, None, tbl, None), EINVAL, "null output")
-    rejected(lib.muon_hip_total_norm(tbl, 0, F32, 0, tbl, tbl, None), EINVAL, "empty list")
-    rejected(lib.muon_hip_total_norm(tbl, 1, F32, 7, tbl, tbl, None), EINVAL, "norm kind")
-    rejected(lib.muon_hip_grad_norms(tbl, tbl, tbl, 1, 1, F32, 3, tbl, tbl, None), EINVAL, "norm kind")
+    rejected(lib.muon_hip_grad_norms(tbl, tbl, None, 1, 1, F32, 2.0, tbl, tbl, None), EINVAL, "null tensor-list")
+    rejected(lib.muon_hip_grad_norms(tbl, tbl, tbl, 1, 1, F32, 2.0, None, tbl, None), EINVAL, "null output")
+    rejected(lib.muon_hip_total_norm(tbl, 0, F32, 2.0, tbl, tbl, None), EINVAL, "empty list")
+    rejected(lib.muon_hip_total_norm(tbl, 1, F32, float("nan"), tbl, tbl, None), EINVAL, "norm_type is NaN")
+    rejected(lib.muon_hip_grad_norms(tbl, tbl, tbl, 1, 1, F32, float("nan"), tbl, tbl, None), EINVAL, "norm_type is NaN")
     rejected(lib.muon_hip_clip_scale(tbl, tbl, tbl, 1, 1, F32, None, F32, 1.0, None), EINVAL, "null total")
     rejected(lib.muon_hip_clip_scale(tbl, tbl, tbl, 1, 1 << 31, F32, tbl, F32, 1.0, None), ESHAPE, "chunks exceed")
     rejected(lib.muon_hip_timing_read(99, None, None), EINVAL, "kernel id")
     rejected(lib.muon_hip_syrk_bf16(tbl, tbl + 64, 512, 512, 1, _abi.CFG_AUTO, tbl + 8, None), EINVAL, "64-byte aligned")
     rejected(lib.muon_hip_timing_reserve(-1), EINVAL, "can be reserved")
-    rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, (1 << 20) + 1, F32, 0, tbl, None), ESHAPE, "built-in scratch")
-    rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, 1, F32, 0, None, None), EINVAL, "null output")
+    rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, (1 << 20) + 1, F32, 2.0, tbl, None), ESHAPE, "built-in scratch")
+    rejected(lib.muon_hip_grad_norms_static(tbl, tbl, tbl, 1, 1, F32, 2.0, None, None), EINVAL, "null output")
 
 
 def test_chunk_choice_lands_on_whole_rounds():

@@ -12,11 +12,11 @@ def _norms(lib, abi, table, dtype, dev, static):
     norms = torch.full((table.n,), float("nan"), dtype=torch.float32, device=dev)
     if static:
         abi.check(lib.muon_hip_grad_norms_static(table.role_ptrs[0], table.numel_ptr, table.chunk_start_ptr, table.n,
-                                                 table.chunks, abi.dtype_code(dtype), abi.NORM_L2, norms.data_ptr(), 0), "static")
+                                                 table.chunks, abi.dtype_code(dtype), 2.0, norms.data_ptr(), 0), "static")
     else:
         partials = torch.full((table.chunks,), float("nan"), dtype=torch.float32, device=dev)
         abi.check(lib.muon_hip_grad_norms(table.role_ptrs[0], table.numel_ptr, table.chunk_start_ptr, table.n,
-                                          table.chunks, abi.dtype_code(dtype), abi.NORM_L2, partials.data_ptr(), norms.data_ptr(), 0),
+                                          table.chunks, abi.dtype_code(dtype), 2.0, partials.data_ptr(), norms.data_ptr(), 0),
                   "caller scratch")
     torch.cuda.synchronize()
     return norms
@@ -43,5 +43,5 @@ def test_static_scratch_entry_point_matches_caller_scratch(dtype):
         assert torch.allclose(a, ref, rtol=1e-2 if dtype == torch.bfloat16 else 1e-5)
     # the limit is enforced before anything is launched
     rc = lib.muon_hip_grad_norms_static(table.role_ptrs[0], table.numel_ptr, table.chunk_start_ptr, table.n,
-                                        abi.STATIC_MAX_CHUNKS + 1, abi.dtype_code(dtype), abi.NORM_L2, a.data_ptr(), 0)
+                                        abi.STATIC_MAX_CHUNKS + 1, abi.dtype_code(dtype), 2.0, a.data_ptr(), 0)
     assert rc == -2 and b"built-in scratch" in lib.muon_hip_last_error()
