@@ -224,24 +224,35 @@ def fast_newtonschulz(G: Tensor, steps: int = 5) -> Tensor:
     return out
 
 
+def _row_major(t: Tensor) -> Tensor:
+    """t itself when its strides are row-major, else a row-major copy (the caller writes it back)."""
+    return t if t.is_contiguous() else t.detach().contiguous()
+
+
 def apply_momentum(grad: Tensor, momentum: Tensor, beta: float, nesterov: bool) -> Tensor:
-    """In place on both tensors, as muon_utils.py:159-164; returns the update."""
+    """In place on both tensors, as muon_utils.py:159-164; returns the update.  Tensors whose strides are not
+    row-major go through row-major copies that are written back."""
     _require_cuda(grad, "grad")
-    g2 = grad.view(len(grad), -1) if grad.ndim == 4 else grad
-    assert g2.ndim == 2 and grad.is_contiguous() and momentum.is_contiguous()
+    gc, mc = _row_major(grad), _row_major(momentum)
+    g2 = gc.view(len(gc), -1) if gc.ndim == 4 else gc
+    assert g2.ndim == 2 and momentum.shape == grad.shape
     rows, cols = g2.shape
     with torch.cuda.device(grad.device):
         ws = _workspace(_abi.workspace_bytes(rows, cols, 1), grad.device)
-        gt, mt = _pointer_table([grad], grad.device), _pointer_table([momentum], grad.device)
+        gt, mt = _pointer_table([gc], grad.device), _pointer_table([mc], grad.device)
         _abi.check(
             _abi.lib().muon_hip_momentum_norm(gt.data_ptr(), mt.data_ptr(), _abi.dtype_code(grad.dtype),
                                               _abi.dtype_code(momentum.dtype), ws.data_ptr(), rows, cols, 1,
                                               float(beta), int(bool(nesterov)), 1, _abi.stream_ptr(grad.device)),
             "momentum_norm",
         )
+        if gc is not grad:
+            grad.copy_(gc)
+        if mc is not momentum:
+            momentum.copy_(mc)
     update = grad if nesterov else momentum
     if update.ndim == 4:
-        update = update.view(len(update), -1)
+        update = update.reshape(len(update), -1)
     return update
 
 
@@ -249,15 +260,16 @@ def apply_scaling(grad: Tensor, rms_scale: bool = False) -> Tensor:
     """muon_utils.py:167-175, in place, one rounding in grad's dtype.  step() fuses this into the update kernel;
     this is the stand-alone helper."""
     _require_cuda(grad, "grad")
-    if not grad.is_contiguous():
-        raise NotImplementedError("apply_scaling needs a contiguous tensor")
+    gc = _row_major(grad)
     with torch.cuda.device(grad.device):
         _abi.check(
-            _abi.lib().muon_hip_scale(grad.data_ptr(), _abi.dtype_code(grad.dtype), grad.numel(),
+            _abi.lib().muon_hip_scale(gc.data_ptr(), _abi.dtype_code(grad.dtype), grad.numel(),
                                       float(scale_factor(grad.size(-2), grad.size(-1), rms_scale)),
                                       _abi.stream_ptr(grad.device)),
             "scale",
         )
+        if gc is not grad:
+            grad.copy_(gc)
     return grad
 
 
@@ -266,17 +278,21 @@ def adam_update(grad: Tensor, buf1: Tensor, buf2: Tensor, step: int, betas, eps:
     _require_cuda(grad, "grad")
     if not (grad.dtype == buf1.dtype == buf2.dtype):
         raise TypeError("adam_update: grad and both moment buffers must share one dtype")
-    if not (buf1.is_contiguous() and buf2.is_contiguous()) or grad.shape != buf1.shape or grad.shape != buf2.shape:
-        raise NotImplementedError("adam_update needs contiguous moment buffers of the gradient's shape")
-    g = grad if grad.is_contiguous() else grad.contiguous()
-    out = torch.empty_like(buf1)
+    if grad.shape != buf1.shape or grad.shape != buf2.shape:
+        raise ValueError("adam_update: the moment buffers must have the gradient's shape")
+    g, b1, b2 = _row_major(grad), _row_major(buf1), _row_major(buf2)
+    out = torch.empty_like(b1)
     with torch.cuda.device(grad.device):
         _abi.check(
-            _abi.lib().muon_hip_adam_update(g.data_ptr(), buf1.data_ptr(), buf2.data_ptr(), out.data_ptr(),
+            _abi.lib().muon_hip_adam_update(g.data_ptr(), b1.data_ptr(), b2.data_ptr(), out.data_ptr(),
                                             _abi.dtype_code(grad.dtype), grad.numel(), int(step), float(betas[0]),
                                             float(betas[1]), float(eps), _abi.stream_ptr(grad.device)),
             "adam_update",
         )
+        if b1 is not buf1:
+            buf1.copy_(b1)
+        if b2 is not buf2:
+            buf2.copy_(b2)
     return out
 
 

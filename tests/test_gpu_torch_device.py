@@ -199,3 +199,43 @@ def test_step_deepspeed_is_the_torch_expressions_on_device(env, pdtype, udtype):
     ref.add_(u.reshape(ref.shape), alpha=-0.02)
     assert torch.equal(p.detach(), ref), _mismatch(p.detach(), ref)
     assert opt.state[q]["step"] == 1 and not torch.equal(q.detach(), e)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_functional_helpers_take_strided_tensors(env, dtype):
+    """The reference's helpers are torch expressions and take tensors of any strides (muon_utils.py:159-183); here
+    such tensors go through row-major copies that are written back, so the views still hold the results."""
+    print(f"strided helpers {dtype}", flush=True)
+    mu, dev = env["mu"], env["dev"]
+    gen = torch.Generator().manual_seed(5)
+    rows, cols, beta = 96, 160, 0.95
+
+    def pair(scale):
+        dense = (scale * torch.randn(rows, cols, generator=gen)).to(dtype).to(dev)
+        wide = torch.zeros(rows, 2 * cols, dtype=dtype, device=dev)
+        view = wide[:, ::2]          # strided with gaps
+        view.copy_(dense)
+        return dense, view
+
+    g, gv = pair(1e-3)
+    m, mt = pair(1e-3)
+    mv = mt.t().contiguous().t()     # dense, column-major
+    assert not gv.is_contiguous() and not mv.is_contiguous()
+    u = mu.apply_momentum(g, m, beta, True)
+    uv = mu.apply_momentum(gv, mv, beta, True)
+    torch.cuda.synchronize()
+    assert uv is gv and torch.equal(uv, u) and torch.equal(mv, m)
+    s, sv = pair(1.0)
+    assert mu.apply_scaling(sv, True) is sv
+    assert torch.equal(sv, mu.apply_scaling(s, True))
+    gr, grv = pair(1e-2)
+    e1, e1v = pair(1e-3)
+    e2, e2v = pair(1e-3)
+    e2.abs_()
+    e2v.abs_()
+    out = mu.adam_update(gr, e1, e2, 3, (0.9, 0.95), 1e-8)
+    outv = mu.adam_update(grv, e1v, e2v, 3, (0.9, 0.95), 1e-8)
+    torch.cuda.synchronize()
+    assert torch.equal(outv, out) and torch.equal(e1v, e1) and torch.equal(e2v, e2)
+    with pytest.raises(ValueError):
+        mu.adam_update(gr, e1[:4], e2, 3, (0.9, 0.95), 1e-8)
