@@ -211,6 +211,10 @@ def fast_newtonschulz(G: Tensor, steps: int = 5) -> Tensor:
     batch = G.size(0) if G.ndim == 3 else 1
     rows, cols = G.size(-2), G.size(-1)
     Gc = G.contiguous()
+    if Gc.dtype in (torch.float16, torch.float64):
+        # G.bfloat16() (muon_utils.py:138) converts these through fp32: fp16 -> fp32 is exact, fp64 -> fp32 is the
+        # rounding torch's own conversion makes first
+        Gc = Gc.float()
     lib = _abi.lib()
     a, b, c = NS_COEFFS
     with torch.cuda.device(G.device):

@@ -336,6 +336,11 @@ def test_newton_schulz_zero_and_scale(env):
     G = torch.randn(128, 384, generator=torch.Generator().manual_seed(5)).to(env["dev"])
     a, b = mu.fast_newtonschulz(G, 5), mu.fast_newtonschulz(G * 4.0, 5)  # power-of-two scale: identical bf16 inputs
     assert rel_fro(a, b) < 2e-2
+    # G.bfloat16() takes any floating dtype (muon_utils.py:138): fp16 and fp64 inputs give what their bf16 image gives
+    H = G.half()
+    assert torch.equal(mu.fast_newtonschulz(H, 5), mu.fast_newtonschulz(H.bfloat16(), 5))
+    D = G.double()
+    assert torch.equal(mu.fast_newtonschulz(D, 5), mu.fast_newtonschulz(D.bfloat16(), 5))
 
 
 def test_newton_schulz_batched_matches_single_bitwise(env):
