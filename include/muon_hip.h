@@ -253,7 +253,8 @@ int muon_hip_device_shape(int* compute_units, int* xcds);
  * duration and launch count of one kernel id since timing was enabled.  The events come from a pool:
  * muon_hip_timing_reserve(n), called while timing is off, makes sure n pairs exist (enabling creates
  * 4096 if there are fewer), so that a timed launch creates nothing and takes no lock.  Launches beyond
- * the pool run untimed; muon_hip_timing_untimed() counts them since timing was enabled. */
+ * the pool, and launches on a stream that is being captured into a graph, run untimed;
+ * muon_hip_timing_untimed() counts them since timing was enabled. */
 int muon_hip_timing_reserve(long launches);
 int muon_hip_timing_enable(int on);
 int muon_hip_timing_read(int kernel_id, double* total_ms, long* launches);

@@ -72,6 +72,12 @@ struct Timed {
     hipStream_t s;
     Timed(int kid, hipStream_t st) : ev(nullptr), s(st) {
         if (!g_timing.load(std::memory_order_acquire)) return;
+        // a launch that is being recorded into a graph has no time of its own: its events would become graph nodes
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+            g_untimed.fetch_add(1, std::memory_order_relaxed);
+            return;
+        }
         const size_t i = g_used.fetch_add(1, std::memory_order_relaxed);
         if (i >= g_pool_size.load(std::memory_order_acquire)) {
             g_untimed.fetch_add(1, std::memory_order_relaxed);

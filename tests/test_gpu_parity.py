@@ -902,9 +902,16 @@ def test_muon_step_replays_from_a_hip_graph(env):
         oa.step()
         ob.step()
     torch.cuda.synchronize()
+    # Per-kernel timing left switched on does not leak event records into the recording: launches under capture go
+    # untimed and are counted as such.
+    abi = env["abi"]
+    abi.timing_enable(True)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         oa.step()
+    assert abi.lib().muon_hip_timing_untimed() > 0
+    assert sum(cnt for _, cnt in abi.timing_read().values()) == 0
+    abi.timing_enable(False)
     for rep in range(4):
         print(f"graph replay {rep}", flush=True)
         graph.replay()
